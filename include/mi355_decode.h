@@ -735,6 +735,94 @@ int32_t mi355_allreduce_oneshot_status(void* comm);
 int32_t mi355_allreduce_oneshot_status_async(void* comm, uint32_t* host_word, void* stream);
 int32_t mi355_allreduce_oneshot_destroy(void* comm);
 
+/*
+ * Decoders with an fp32 residual stream (no counterpart in the reference: the engine it launches
+ * keeps the residual in the model's 16-bit type).  `dtype` is the storage type of activations and
+ * weights: MI355_BF16, MI355_F16 or MI355_F32; sums, means and transcendentals are fp32 always.
+ *   embed_scale_f32       resid[t] = embed[ids[t]] * scale
+ *   resid_add_f32         resid[t] += other[t] (fp32, may be null) + vec (one row, may be null)
+ *   add_rms_norm_f32      resid += add (may be null); out = resid / sqrt(mean(resid^2) + eps) * w,
+ *                         w one number (weight_numel 1) or one per column (weight_numel == width)
+ *   rms_norm_mix_f32      resid += alpha * (rmsnorm(xa) * wa + rmsnorm(xb) * wb); xb / wb may be null
+ *   gelu_tanh_and_mul     out[t] = gelu_tanh(x[t, :inter]) * x[t, inter:2 inter]
+ *   gated_head_rms_norm   out[t, h] = o[t, h] / rms(o[t, h]) * weight * act(gate[t, h]); o fp32
+ *                         [tokens, heads, head_dim]; activation 0: silu, 1: sigmoid
+ *   softcap               z = cap * tanh(z / cap), in place
+ */
+int32_t mi355_embed_scale_f32(float* out, const void* embed, const int64_t* ids, int64_t num_tokens,
+                              int32_t width, int64_t vocab, float scale, int32_t dtype, void* stream);
+int32_t mi355_resid_add_f32(float* resid, const float* other, const void* vec, int64_t num_tokens,
+                            int32_t width, int32_t dtype, void* stream);
+int32_t mi355_add_rms_norm_f32(void* out, float* resid, const void* add, const void* weight,
+                               int32_t weight_numel, int64_t num_tokens, int32_t width, float eps,
+                               int32_t dtype, void* stream);
+int32_t mi355_rms_norm_mix_f32(float* resid, const void* xa, const void* wa, const void* xb,
+                               const void* wb, int64_t num_tokens, int32_t width, float eps,
+                               float alpha, int32_t dtype, void* stream);
+int32_t mi355_gelu_tanh_and_mul(void* out, const void* x, int64_t x_stride, int64_t num_tokens,
+                                int32_t inter, int32_t dtype, void* stream);
+int32_t mi355_gated_head_rms_norm(void* out, const float* o, const void* gate, int64_t gate_stride,
+                                  const float* weight, int64_t num_tokens, int32_t num_heads,
+                                  int32_t head_dim, float eps, int32_t activation, int32_t dtype,
+                                  void* stream);
+int32_t mi355_softcap(void* z, int64_t numel, float cap, int32_t dtype, void* stream);
+
+/*
+ * Sequence mixers over a packed batch of chunks (whole prompts, portions of prompts and single
+ * decoded tokens side by side): tok_seq[t] names the chunk of packed row t, positions[t] its
+ * position in its sequence, cu_seqlens[s] the first row of chunk s.  K pages are
+ * [blocks, kv_heads, 16, head_dim], V pages [blocks, kv_heads, 16, v_dim]; convolution state is
+ * fp32 [slots, taps - 1, channels], delta-rule state fp32 [slots, heads, head_dim, v_dim].
+ *   rope_partial_kv_write  rotates the first rot_dims coordinates of every q and k head (coordinate
+ *                          i with i + rot_dims / 2) by the fp32 table cos_sin [max_pos, rot_dims]
+ *                          (cos | sin), q in place, k into its page; v is copied into its page;
+ *                          rows with slot < 0 store nothing
+ *   sigmoid_window_attn    out[t, h] = sigmoid(gate[t, h]) * sum over keys j of the row's sequence with
+ *                          0 <= p - j < window of sigmoid(q.k_j * scale * temp[h] + bias[h]) * v_j
+ *                          (gate may be null); weights are not normalised over keys
+ *   causal_conv_silu       y[t, c] = silu(sum_j w[c, j] * x[t - (taps - 1 - j), c]); inputs from before
+ *                          the chunk come from the sequence's state slot, zeros before position 0
+ *   conv_state_update      state slot <- the last taps - 1 inputs of each sequence (after the conv)
+ *   gated_delta_rule       per token and head, on state S [head_dim, v_dim] (zero at position 0):
+ *                          S <- a S; u = b (v - S^T k); S <- S + k u^T; o = S^T q, with k and q made
+ *                          unit vectors (q also / sqrt(head_dim)), b = sigmoid(beta),
+ *                          a = exp(-exp(a_log[h]) * softplus(decay + dt_bias)), one per head
+ *                          (per_channel 0) or one per key channel (per_channel 1: decay rows
+ *                          [heads * head_dim]); q / k / v are columns q_off / k_off / v_off of qkv rows
+ */
+int32_t mi355_rope_partial_kv_write(void* q, int64_t q_stride, const void* k, int64_t k_stride,
+                                    const void* v, int64_t v_stride, const float* cos_sin,
+                                    int32_t max_pos, const int64_t* positions,
+                                    const int64_t* slot_mapping, void* k_cache, void* v_cache,
+                                    int64_t num_tokens, int32_t num_heads, int32_t num_kv_heads,
+                                    int32_t head_dim, int32_t v_dim, int32_t rot_dims, int32_t dtype,
+                                    void* stream);
+int32_t mi355_sigmoid_window_attn(void* out, const void* q, int64_t q_stride, const void* k_cache,
+                                  const void* v_cache, const int32_t* block_tables,
+                                  int32_t max_blocks, const int32_t* tok_seq,
+                                  const int64_t* positions, const float* temp, const float* bias,
+                                  const void* gate, int64_t gate_stride, int64_t num_tokens,
+                                  int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
+                                  int32_t v_dim, int32_t window, float scale, int32_t dtype,
+                                  void* stream);
+int32_t mi355_causal_conv_silu(void* y, const void* x, int64_t x_stride, const void* weight,
+                               const float* state, const int32_t* tok_seq, const int64_t* positions,
+                               const int32_t* cu_seqlens, const int32_t* state_slots,
+                               int64_t num_tokens, int32_t channels, int32_t taps, int32_t dtype,
+                               void* stream);
+int32_t mi355_conv_state_update(float* state, const void* x, int64_t x_stride,
+                                const int32_t* cu_seqlens, const int32_t* state_slots,
+                                int32_t num_seqs, int32_t channels, int32_t taps, int32_t dtype,
+                                void* stream);
+int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t stride, int32_t q_off,
+                               int32_t k_off, int32_t v_off, const void* beta, int64_t beta_stride,
+                               const void* decay, int64_t decay_stride, const float* a_log,
+                               const float* dt_bias, int32_t per_channel, float* state,
+                               const int32_t* cu_seqlens, const int64_t* positions,
+                               const int32_t* state_slots, int32_t num_seqs, int32_t num_heads,
+                               int32_t num_kv_heads, int32_t head_dim, int32_t v_dim, int32_t dtype,
+                               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

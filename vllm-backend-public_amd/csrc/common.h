@@ -220,6 +220,40 @@ __device__ __forceinline__ void bounds_store(const void* base, void* p, const W&
 #define MI355_OK_AT(base, p, bytes) true
 #endif
 
+// ---- element access for kernels that keep some tensors in 32 bits --------------------------------
+// F32 joins BF16 / F16 as a storage type for the kernels whose arithmetic is fp32 throughout and
+// whose activations may be stored in 16 or in 32 bits (the residual stream, recurrent state and
+// every reduction of those kernels are fp32 whatever the storage type is).
+struct F32 {};
+template <typename T> struct Elem { typedef uint16_t S; };
+template <> struct Elem<F32> { typedef float S; };
+template <typename T>
+__device__ __forceinline__ float elem_to_f(typename Elem<T>::S v) { return T::to_f(v); }
+template <>
+__device__ __forceinline__ float elem_to_f<F32>(float v) { return v; }
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::S elem_from_f(float f) { return T::from_f(f); }
+template <>
+__device__ __forceinline__ float elem_from_f<F32>(float f) { return f; }
+#define MI355_LDF(T, base, p) (::mi355::elem_to_f<T>(MI355_LD(typename ::mi355::Elem<T>::S, (base), (p))))
+#define MI355_STF(T, base, p, f) MI355_ST(typename ::mi355::Elem<T>::S, (base), (p), ::mi355::elem_from_f<T>(f))
+// dispatch on an mi355_dtype code: BODY sees the storage type as TT
+#define MI355_DISPATCH_DTYPE3(dtype, ...)                                   \
+  do {                                                                      \
+    if ((dtype) == MI355_BF16) { typedef ::mi355::BF16 TT; __VA_ARGS__; }   \
+    else if ((dtype) == MI355_F16) { typedef ::mi355::F16 TT; __VA_ARGS__; } \
+    else { typedef ::mi355::F32 TT; __VA_ARGS__; }                          \
+  } while (0)
+__device__ __forceinline__ float block_sum32(float v, float* scratch /* >= 32 floats of LDS */) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+  __syncthreads();                                  // scratch may still be read from a previous call
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nw; ++i) t += scratch[i];
+  return t;
+}
 // ---- host side ------------------------------------------------------------
 int32_t fail(int32_t code, const char* fmt, ...);
 

@@ -1,0 +1,260 @@
+// Pointwise and normalisation kernels for decoders that keep the residual stream in fp32:
+//   embed_scale_f32          resid = embed[id] * scale
+//   resid_add_f32            resid += other (fp32 rows) + vec (one row, broadcast)
+//   add_rms_norm_f32         resid += add; out = resid / rms(resid) * w      (w: one number or a vector)
+//   rms_norm_mix_f32         resid += alpha * (xa / rms(xa) * wa + xb / rms(xb) * wb)
+//   gelu_tanh_and_mul        out = gelu_tanh(gate) * up for rows holding gate | up
+//   gated_head_rms_norm      out = o / rms(o) * w * act(gate) per (token, head) row of an fp32 tensor
+//   softcap                  z = cap * tanh(z / cap)
+// Every sum, mean and transcendental is fp32; activations are stored in bf16, fp16 or fp32
+// (the dtype argument).  HBM-bound: one pass over the rows, one workgroup (or one wave) per row.
+#include "common.h"
+
+namespace mi355 {
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_scale_f32_kernel(float* __restrict__ out,
+                                                              const typename Elem<T>::S* __restrict__ embed,
+                                                              const int64_t* __restrict__ ids, int W, float scale) {
+  const int64_t t = blockIdx.x;
+  const int64_t id = MI355_LD(int64_t, ids, ids + t);
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    MI355_ST(float, out, out + t * W + c, MI355_LDF(T, embed, embed + id * W + c) * scale);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void resid_add_f32_kernel(float* __restrict__ resid, const float* __restrict__ other,
+                                                            const typename Elem<T>::S* __restrict__ vec, int W) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = MI355_LD(float, resid, resid + t * W + c);
+    if (other != nullptr) v += MI355_LD(float, other, other + t * W + c);
+    if (vec != nullptr) v += MI355_LDF(T, vec, vec + c);
+    MI355_ST(float, resid, resid + t * W + c, v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void add_rms_norm_f32_kernel(typename Elem<T>::S* __restrict__ out,
+                                                               float* __restrict__ resid,
+                                                               const typename Elem<T>::S* __restrict__ add,
+                                                               const typename Elem<T>::S* __restrict__ weight,
+                                                               int weight_numel, int W, float eps) {
+  __shared__ float scratch[32];
+  const int64_t t = blockIdx.x;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = MI355_LD(float, resid, resid + t * W + c);
+    if (add != nullptr) {
+      v += MI355_LDF(T, add, add + t * W + c);
+      MI355_ST(float, resid, resid + t * W + c, v);
+    }
+    ss += v * v;
+  }
+  ss = block_sum32(ss, scratch);
+  const float r = 1.0f / sqrtf(ss / static_cast<float>(W) + eps);
+  const float g1 = weight_numel == 1 ? MI355_LDF(T, weight, weight) : 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = MI355_LD(float, resid, resid + t * W + c);      // own writes of this thread: same c
+    const float g = weight_numel == 1 ? g1 : MI355_LDF(T, weight, weight + c);
+    MI355_STF(T, out, out + t * W + c, v * r * g);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_mix_f32_kernel(float* __restrict__ resid,
+                                                               const typename Elem<T>::S* __restrict__ xa,
+                                                               const typename Elem<T>::S* __restrict__ wa,
+                                                               const typename Elem<T>::S* __restrict__ xb,
+                                                               const typename Elem<T>::S* __restrict__ wb, int W,
+                                                               float eps, float alpha) {
+  __shared__ float scratch[32];
+  const int64_t t = blockIdx.x;
+  float sa = 0.f, sb = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float a = MI355_LDF(T, xa, xa + t * W + c);
+    sa += a * a;
+    if (xb != nullptr) {
+      const float b = MI355_LDF(T, xb, xb + t * W + c);
+      sb += b * b;
+    }
+  }
+  sa = block_sum32(sa, scratch);
+  sb = block_sum32(sb, scratch);
+  const float ra = 1.0f / sqrtf(sa / static_cast<float>(W) + eps);
+  const float rb = 1.0f / sqrtf(sb / static_cast<float>(W) + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float m = MI355_LDF(T, xa, xa + t * W + c) * ra * MI355_LDF(T, wa, wa + c);
+    if (xb != nullptr) m += MI355_LDF(T, xb, xb + t * W + c) * rb * MI355_LDF(T, wb, wb + c);
+    const float v = MI355_LD(float, resid, resid + t * W + c);
+    MI355_ST(float, resid, resid + t * W + c, v + alpha * m);
+  }
+}
+
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_tanh_and_mul_kernel(typename Elem<T>::S* __restrict__ out,
+                                                                const typename Elem<T>::S* __restrict__ x,
+                                                                int64_t x_stride, int64_t num_tokens, int inter) {
+  const int64_t total = num_tokens * inter;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t row = i / inter;
+    const int c = static_cast<int>(i % inter);
+    const float g = MI355_LDF(T, x, x + row * x_stride + c);
+    const float u = MI355_LDF(T, x, x + row * x_stride + inter + c);
+    MI355_STF(T, out, out + row * inter + c, gelu_tanh_f(g) * u);
+  }
+}
+
+// one wave per (token, head) row of o [rows = T * H][dv]
+template <typename T>
+__global__ __launch_bounds__(256) void gated_head_rms_norm_kernel(typename Elem<T>::S* __restrict__ out,
+                                                                  const float* __restrict__ o,
+                                                                  const typename Elem<T>::S* __restrict__ gate,
+                                                                  int64_t gate_stride, const float* __restrict__ w,
+                                                                  int64_t rows, int H, int dv, float eps, int act) {
+  const int64_t row = blockIdx.x * static_cast<int64_t>(blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = row / H;
+  const int h = static_cast<int>(row % H);
+  float ss = 0.f;
+  for (int c = lane; c < dv; c += 64) {
+    const float v = MI355_LD(float, o, o + row * dv + c);
+    ss += v * v;
+  }
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / static_cast<float>(dv) + eps);
+  for (int c = lane; c < dv; c += 64) {
+    const float v = MI355_LD(float, o, o + row * dv + c);
+    const float g = MI355_LDF(T, gate, gate + t * gate_stride + static_cast<int64_t>(h) * dv + c);
+    const float s = 1.0f / (1.0f + expf(-g));
+    const float a = act == 0 ? g * s : s;
+    MI355_STF(T, out, out + row * dv + c, v * r * MI355_LD(float, w, w + c) * a);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softcap_kernel(typename Elem<T>::S* __restrict__ z, int64_t n, float cap) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    MI355_STF(T, z, z + i, cap * tanhf(MI355_LDF(T, z, z + i) / cap));
+}
+
+static inline dim3 stride_grid(int64_t total) {
+  const int64_t blocks = (total + 255) / 256;
+  return dim3(static_cast<unsigned>(blocks < 1 ? 1 : (blocks > 65536 ? 65536 : blocks)));
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+#define REQ_DTYPE(dtype) MI355_REQUIRE((dtype) >= MI355_BF16 && (dtype) <= MI355_F32, MI355_ERR_UNSUPPORTED, "dtype code %d", (dtype))
+
+extern "C" int32_t mi355_embed_scale_f32(float* out, const void* embed, const int64_t* ids, int64_t num_tokens,
+                                         int32_t width, int64_t vocab, float scale, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && embed && ids, MI355_ERR_INVALID, "embed_scale_f32: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && width > 0 && vocab > 0, MI355_ERR_INVALID, "embed_scale_f32: sizes");
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((embed_scale_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s, out,
+                                                  static_cast<const Elem<TT>::S*>(embed), ids, width, scale));
+  return check_launch("embed_scale_f32");
+}
+
+extern "C" int32_t mi355_resid_add_f32(float* resid, const float* other, const void* vec, int64_t num_tokens,
+                                       int32_t width, int32_t dtype, void* stream) {
+  MI355_REQUIRE(resid, MI355_ERR_INVALID, "resid_add_f32: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && width > 0, MI355_ERR_INVALID, "resid_add_f32: sizes");
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0 || (!other && !vec)) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((resid_add_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s, resid,
+                                                  other, static_cast<const Elem<TT>::S*>(vec), width));
+  return check_launch("resid_add_f32");
+}
+
+extern "C" int32_t mi355_add_rms_norm_f32(void* out, float* resid, const void* add, const void* weight,
+                                          int32_t weight_numel, int64_t num_tokens, int32_t width, float eps,
+                                          int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && resid && weight, MI355_ERR_INVALID, "add_rms_norm_f32: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && width > 0, MI355_ERR_INVALID, "add_rms_norm_f32: sizes");
+  MI355_REQUIRE(weight_numel == 1 || weight_numel == width, MI355_ERR_INVALID,
+                "add_rms_norm_f32: the weight is one number or one per column (%d for width %d)", weight_numel, width);
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((add_rms_norm_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), resid,
+                                                  static_cast<const Elem<TT>::S*>(add),
+                                                  static_cast<const Elem<TT>::S*>(weight), weight_numel, width, eps));
+  return check_launch("add_rms_norm_f32");
+}
+
+extern "C" int32_t mi355_rms_norm_mix_f32(float* resid, const void* xa, const void* wa, const void* xb, const void* wb,
+                                          int64_t num_tokens, int32_t width, float eps, float alpha, int32_t dtype,
+                                          void* stream) {
+  MI355_REQUIRE(resid && xa && wa && ((xb == nullptr) == (wb == nullptr)), MI355_ERR_INVALID,
+                "rms_norm_mix_f32: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && width > 0, MI355_ERR_INVALID, "rms_norm_mix_f32: sizes");
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((rms_norm_mix_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s, resid,
+                                                  static_cast<const Elem<TT>::S*>(xa), static_cast<const Elem<TT>::S*>(wa),
+                                                  static_cast<const Elem<TT>::S*>(xb), static_cast<const Elem<TT>::S*>(wb),
+                                                  width, eps, alpha));
+  return check_launch("rms_norm_mix_f32");
+}
+
+extern "C" int32_t mi355_gelu_tanh_and_mul(void* out, const void* x, int64_t x_stride, int64_t num_tokens,
+                                           int32_t inter, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && x, MI355_ERR_INVALID, "gelu_tanh_and_mul: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && inter > 0 && x_stride >= 2 * static_cast<int64_t>(inter), MI355_ERR_INVALID,
+                "gelu_tanh_and_mul: sizes");
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((gelu_tanh_and_mul_kernel<TT>), stride_grid(num_tokens * inter), dim3(256),
+                                                  0, s, static_cast<Elem<TT>::S*>(out),
+                                                  static_cast<const Elem<TT>::S*>(x), x_stride, num_tokens, inter));
+  return check_launch("gelu_tanh_and_mul");
+}
+
+extern "C" int32_t mi355_gated_head_rms_norm(void* out, const float* o, const void* gate, int64_t gate_stride,
+                                             const float* weight, int64_t num_tokens, int32_t num_heads,
+                                             int32_t head_dim, float eps, int32_t activation, int32_t dtype,
+                                             void* stream) {
+  MI355_REQUIRE(out && o && gate && weight, MI355_ERR_INVALID, "gated_head_rms_norm: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && num_heads > 0 && head_dim > 0 &&
+                    gate_stride >= static_cast<int64_t>(num_heads) * head_dim,
+                MI355_ERR_INVALID, "gated_head_rms_norm: sizes");
+  MI355_REQUIRE(activation == 0 || activation == 1, MI355_ERR_INVALID,
+                "gated_head_rms_norm: activation is 0 (silu) or 1 (sigmoid)");
+  REQ_DTYPE(dtype);
+  const int64_t rows = num_tokens * num_heads;
+  if (rows == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((gated_head_rms_norm_kernel<TT>), dim3((rows + 3) / 4), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), o,
+                                                  static_cast<const Elem<TT>::S*>(gate), gate_stride, weight, rows,
+                                                  num_heads, head_dim, eps, activation));
+  return check_launch("gated_head_rms_norm");
+}
+
+extern "C" int32_t mi355_softcap(void* z, int64_t numel, float cap, int32_t dtype, void* stream) {
+  MI355_REQUIRE(z, MI355_ERR_INVALID, "softcap: null pointer");
+  MI355_REQUIRE(numel >= 0 && cap > 0.f, MI355_ERR_INVALID, "softcap: sizes");
+  REQ_DTYPE(dtype);
+  if (numel == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((softcap_kernel<TT>), stride_grid(numel), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(z), numel, cap));
+  return check_launch("softcap");
+}

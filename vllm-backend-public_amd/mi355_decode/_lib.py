@@ -96,6 +96,21 @@ def _load() -> ctypes.CDLL:
         "mi355_allreduce_oneshot_status_async": (I32, [P, P, P]),
         "mi355_allreduce_oneshot_destroy": (I32, [P]),
         "mi355_linear_decode": (I32, [P, I64, P, I64, P, P, I32, I32, I32, I32, I32, P]),
+        "mi355_embed_scale_f32": (I32, [P, P, P, I64, I32, I64, F, I32, P]),
+        "mi355_resid_add_f32": (I32, [P, P, P, I64, I32, I32, P]),
+        "mi355_add_rms_norm_f32": (I32, [P, P, P, P, I32, I64, I32, F, I32, P]),
+        "mi355_rms_norm_mix_f32": (I32, [P, P, P, P, P, I64, I32, F, F, I32, P]),
+        "mi355_gelu_tanh_and_mul": (I32, [P, P, I64, I64, I32, I32, P]),
+        "mi355_gated_head_rms_norm": (I32, [P, P, P, I64, P, I64, I32, I32, F, I32, I32, P]),
+        "mi355_softcap": (I32, [P, I64, F, I32, P]),
+        "mi355_rope_partial_kv_write": (I32, [P, I64, P, I64, P, I64, P, I32, P, P, P, P, I64, I32, I32, I32, I32, I32,
+                                              I32, P]),
+        "mi355_sigmoid_window_attn": (I32, [P, P, I64, P, P, P, I32, P, P, P, P, P, I64, I64, I32, I32, I32, I32, I32,
+                                            F, I32, P]),
+        "mi355_causal_conv_silu": (I32, [P, P, I64, P, P, P, P, P, P, I64, I32, I32, I32, P]),
+        "mi355_conv_state_update": (I32, [P, P, I64, P, P, I32, I32, I32, I32, P]),
+        "mi355_gated_delta_rule": (I32, [P, P, I64, I32, I32, I32, P, I64, P, I64, P, P, I32, P, P, P, P, I32, I32, I32,
+                                         I32, I32, I32, P]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
@@ -125,7 +140,11 @@ EXPORTS = ("mi355_abi_version", "mi355_last_error", "mi355_target_arch",
            "mi355_allreduce_oneshot_handle_bytes", "mi355_allreduce_oneshot_init", "mi355_allreduce_oneshot_connect",
            "mi355_allreduce_oneshot_run", "mi355_allreduce_oneshot_run_slabs", "mi355_allreduce_oneshot_run_add_norm", "mi355_allreduce_twoshot_run_add_norm", "mi355_allreduce_oneshot_run_max_keys",
            "mi355_allreduce_oneshot_status",
-           "mi355_allreduce_oneshot_status_async", "mi355_allreduce_oneshot_destroy")
+           "mi355_allreduce_oneshot_status_async", "mi355_allreduce_oneshot_destroy",
+           "mi355_embed_scale_f32", "mi355_resid_add_f32", "mi355_add_rms_norm_f32", "mi355_rms_norm_mix_f32",
+           "mi355_gelu_tanh_and_mul", "mi355_gated_head_rms_norm", "mi355_softcap",
+           "mi355_rope_partial_kv_write", "mi355_sigmoid_window_attn", "mi355_causal_conv_silu",
+           "mi355_conv_state_update", "mi355_gated_delta_rule")
 
 
 def check(status: int) -> None:

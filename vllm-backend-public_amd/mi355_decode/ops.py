@@ -916,3 +916,237 @@ def linear_tiled_w8a8(xq: torch.Tensor, x_scale: torch.Tensor, w_fp8: torch.Tens
                                       w_fp8.data_ptr(), w_scale.data_ptr(), bias.data_ptr() if bias is not None else 0,
                                       M, N, K, tiles_per_wg, k_groups, epilogue, dt, _stream()))
     return ret
+
+
+# ---------------------------------------------------------------------------------------------- #
+# decoders with an fp32 residual stream; sequence mixers over packed chunks (csrc/resid32.hip,
+# csrc/seqmix.hip).  Activations and weights are bf16, fp16 or fp32; the residual, recurrent
+# state and the small per-head parameters are fp32 tensors.
+# ---------------------------------------------------------------------------------------------- #
+def _dt3(t: torch.Tensor, name: str) -> int:
+    _dev(t, name)
+    if t.dtype not in _DT:
+        raise TypeError(f"{name}: dtype {t.dtype} not supported (bfloat16/float16/float32)")
+    return _DT[t.dtype]
+
+
+def _f32(t: torch.Tensor, name: str, numel: int | None = None) -> int:
+    _dev(t, name)
+    if t.dtype != torch.float32 or not t.is_contiguous() or (numel is not None and t.numel() != numel):
+        raise ValueError(f"{name} must be a contiguous float32 tensor" + (f" of {numel} elements" if numel else ""))
+    return t.data_ptr()
+
+
+def _idx(t: torch.Tensor, name: str, dtype: torch.dtype, numel: int | None = None) -> int:
+    _dev(t, name)
+    if t.dtype != dtype or not t.is_contiguous() or (numel is not None and t.numel() < numel):
+        raise ValueError(f"{name} must be a contiguous {dtype} tensor" + (f" of >= {numel} elements" if numel else ""))
+    return t.data_ptr()
+
+
+def _same(t: torch.Tensor, ref: torch.Tensor, name: str) -> int:
+    _dev(t, name)
+    if t.dtype != ref.dtype:
+        raise TypeError(f"{name}: dtype {t.dtype}, expected {ref.dtype}")
+    return t.data_ptr()
+
+
+def embed_scale_f32(embed: torch.Tensor, ids: torch.Tensor, scale: float, out: torch.Tensor | None = None):
+    """out[t] = embed[ids[t]] * scale as float32 rows."""
+    dt = _dt3(embed, "embed")
+    if embed.dim() != 2 or not embed.is_contiguous():
+        raise ValueError("embed must be contiguous [vocab, width]")
+    T, W = ids.numel(), embed.shape[1]
+    if out is None:
+        out = torch.empty(T, W, dtype=torch.float32, device=embed.device)
+    check(lib.mi355_embed_scale_f32(_f32(out, "out", T * W), embed.data_ptr(), _idx(ids, "ids", torch.int64), T, W,
+                                    embed.shape[0], float(scale), dt, _stream()))
+    return out
+
+
+def resid_add_f32(resid: torch.Tensor, other: torch.Tensor | None = None, vec: torch.Tensor | None = None):
+    """resid += other (float32 rows) + vec (one row of any supported dtype), in place."""
+    T, W = resid.shape
+    dt = _DT[torch.float32]
+    if vec is not None:
+        dt = _dt3(vec, "vec")
+        if vec.numel() != W or not vec.is_contiguous():
+            raise ValueError("vec must be one contiguous row of the residual's width")
+    check(lib.mi355_resid_add_f32(_f32(resid, "resid"), None if other is None else _f32(other, "other", T * W),
+                                  None if vec is None else vec.data_ptr(), T, W, dt, _stream()))
+    return resid
+
+
+def add_rms_norm_f32(resid: torch.Tensor, weight: torch.Tensor, eps: float, add: torch.Tensor | None = None,
+                     out: torch.Tensor | None = None):
+    """resid (float32, in place) += add; returns resid / rms(resid) * weight in the dtype of weight.
+    weight: one number (numel 1) or one per column."""
+    T, W = resid.shape
+    dt = _dt3(weight, "weight")
+    if weight.numel() not in (1, W) or not weight.is_contiguous():
+        raise ValueError("weight must be one number or one contiguous row")
+    if out is None:
+        out = torch.empty(T, W, dtype=weight.dtype, device=resid.device)
+    if out.dtype != weight.dtype or not out.is_contiguous() or out.shape != resid.shape:
+        raise ValueError("out must be contiguous, shaped like resid, in the dtype of weight")
+    if add is not None and (add.dtype != weight.dtype or not add.is_contiguous() or add.shape != resid.shape):
+        raise ValueError("add must be contiguous, shaped like resid, in the dtype of weight")
+    check(lib.mi355_add_rms_norm_f32(out.data_ptr(), _f32(resid, "resid"), None if add is None else add.data_ptr(),
+                                     weight.data_ptr(), weight.numel(), T, W, float(eps), dt, _stream()))
+    return out
+
+
+def rms_norm_mix_f32(resid: torch.Tensor, xa: torch.Tensor, wa: torch.Tensor, xb: torch.Tensor | None,
+                     wb: torch.Tensor | None, eps: float, alpha: float):
+    """resid (float32, in place) += alpha * (rmsnorm(xa) * wa + rmsnorm(xb) * wb)."""
+    T, W = resid.shape
+    dt = _dt3(xa, "xa")
+    for n, t, shape in (("xa", xa, (T, W)), ("wa", wa, (W,)), ("xb", xb, (T, W)), ("wb", wb, (W,))):
+        if t is None:
+            continue
+        if t.dtype != xa.dtype or not t.is_contiguous() or tuple(t.shape) != shape:
+            raise ValueError(f"{n} must be contiguous {shape} in the dtype of xa")
+    check(lib.mi355_rms_norm_mix_f32(_f32(resid, "resid"), xa.data_ptr(), wa.data_ptr(),
+                                     None if xb is None else xb.data_ptr(), None if wb is None else wb.data_ptr(),
+                                     T, W, float(eps), float(alpha), dt, _stream()))
+    return resid
+
+
+def gelu_tanh_and_mul(x: torch.Tensor, out: torch.Tensor | None = None):
+    """x [tokens, 2 * inter] holding gate | up -> gelu_tanh(gate) * up."""
+    dt = _dt3(x, "x")
+    inter = x.shape[1] // 2
+    if out is None:
+        out = torch.empty(x.shape[0], inter, dtype=x.dtype, device=x.device)
+    check(lib.mi355_gelu_tanh_and_mul(out.data_ptr(), x.data_ptr(), _rows(x, "x"), x.shape[0], inter, dt, _stream()))
+    return out
+
+
+ACT_SILU, ACT_SIGMOID = 0, 1
+
+
+def gated_head_rms_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, activation: int,
+                        out: torch.Tensor | None = None):
+    """o float32 [tokens, heads, dim]; gate [tokens, >= heads * dim] (a column slice is fine);
+    weight float32 [dim].  Returns o / rms(o) * weight * act(gate) as [tokens, heads * dim] in gate's dtype."""
+    T, H, D = o.shape
+    dt = _dt3(gate, "gate")
+    if gate.dim() != 2 or gate.shape[1] != H * D or gate.stride(1) != 1:
+        raise ValueError("gate must be [tokens, heads * dim] with a contiguous last dim")
+    if out is None:
+        out = torch.empty(T, H * D, dtype=gate.dtype, device=o.device)
+    check(lib.mi355_gated_head_rms_norm(out.data_ptr(), _f32(o, "o"), gate.data_ptr(), gate.stride(0) if T > 1 else H * D,
+                                        _f32(weight, "weight", D), T, H, D, float(eps), int(activation), dt,
+                                        _stream()))
+    return out
+
+
+def softcap(z: torch.Tensor, cap: float):
+    """z <- cap * tanh(z / cap), in place."""
+    dt = _dt3(z, "z")
+    if not z.is_contiguous():
+        raise ValueError("z must be contiguous")
+    check(lib.mi355_softcap(z.data_ptr(), z.numel(), float(cap), dt, _stream()))
+    return z
+
+
+def _cols(t: torch.Tensor, name: str, width: int) -> int:
+    """Row stride of a [rows, width] column slice."""
+    if t.dim() != 2 or t.shape[1] != width or t.stride(1) != 1:
+        raise ValueError(f"{name} must be [rows, {width}] with a contiguous last dim (shape {tuple(t.shape)})")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), width)
+
+
+def rope_partial_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos_sin: torch.Tensor,
+                          positions: torch.Tensor, slot_mapping: torch.Tensor, k_cache: torch.Tensor,
+                          v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, v_dim: int):
+    """Rotates q in place and k into its page by the float32 table cos_sin [max_pos, rot_dims]; copies v
+    into its page.  q / k / v may be column slices of one projection output."""
+    dt = _dt3(q, "q")
+    T = q.shape[0]
+    rot = cos_sin.shape[1]
+    if tuple(k_cache.shape[1:]) != (num_kv_heads, BLOCK_SIZE, head_dim) or tuple(v_cache.shape[1:]) != (num_kv_heads, BLOCK_SIZE, v_dim) \
+            or k_cache.shape[0] != v_cache.shape[0] or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise ValueError("K pages must be [blocks, kv_heads, 16, head_dim] and V pages [blocks, kv_heads, 16, v_dim]")
+    check(lib.mi355_rope_partial_kv_write(
+        q.data_ptr(), _cols(q, "q", num_heads * head_dim), _same(k, q, "k"), _cols(k, "k", num_kv_heads * head_dim),
+        _same(v, q, "v"), _cols(v, "v", num_kv_heads * v_dim), _f32(cos_sin, "cos_sin"), cos_sin.shape[0],
+        _idx(positions, "positions", torch.int64, T), _idx(slot_mapping, "slot_mapping", torch.int64, T),
+        _same(k_cache, q, "k_cache"), _same(v_cache, q, "v_cache"), T, num_heads, num_kv_heads, head_dim, v_dim, rot,
+        dt, _stream()))
+
+
+def sigmoid_window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                        tok_seq: torch.Tensor, positions: torch.Tensor, temp: torch.Tensor, bias: torch.Tensor,
+                        gate: torch.Tensor | None, num_heads: int, window: int, scale: float,
+                        out: torch.Tensor | None = None):
+    """Sliding-window attention with sigmoid weights over the paged K/V of each packed row's
+    sequence.  Returns [tokens, heads * v_dim]."""
+    dt = _dt3(q, "q")
+    T = q.shape[0]
+    G, d, dv = k_cache.shape[1], k_cache.shape[3], v_cache.shape[3]
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be contiguous int32 [chunks, max_blocks]")
+    if out is None:
+        out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
+    check(lib.mi355_sigmoid_window_attn(
+        out.data_ptr(), q.data_ptr(), _cols(q, "q", num_heads * d), _same(k_cache, q, "k_cache"),
+        _same(v_cache, q, "v_cache"), block_tables.data_ptr(), block_tables.shape[1],
+        _idx(tok_seq, "tok_seq", torch.int32, T), _idx(positions, "positions", torch.int64, T),
+        _f32(temp, "temp", num_heads), _f32(bias, "bias", num_heads),
+        None if gate is None else _same(gate, q, "gate"), 0 if gate is None else _cols(gate, "gate", num_heads),
+        T, num_heads, G, d, dv, int(window), float(scale), dt, _stream()))
+    return out
+
+
+def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, tok_seq: torch.Tensor,
+                     positions: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor,
+                     out: torch.Tensor | None = None):
+    """Depthwise causal convolution + SiLU over packed chunks, then the state update: state
+    [slots, taps - 1, channels] float32 holds each sequence's last taps - 1 inputs."""
+    dt = _dt3(x, "x")
+    T, C = x.shape
+    taps = weight.shape[1]
+    if tuple(weight.shape) != (C, taps) or weight.dtype != x.dtype or not weight.is_contiguous():
+        raise ValueError("weight must be contiguous [channels, taps] in the dtype of x")
+    if state.dim() != 3 or tuple(state.shape[1:]) != (max(taps - 1, 0), C):
+        raise ValueError("state must be [slots, taps - 1, channels]")
+    S = cu_seqlens.numel() - 1
+    if out is None:
+        out = torch.empty(T, C, dtype=x.dtype, device=x.device)
+    args = (_idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(state_slots, "state_slots", torch.int32, S))
+    check(lib.mi355_causal_conv_silu(out.data_ptr(), x.data_ptr(), _cols(x, "x", C), weight.data_ptr(),
+                                     _f32(state, "state"), _idx(tok_seq, "tok_seq", torch.int32, T),
+                                     _idx(positions, "positions", torch.int64, T), *args, T, C, taps, dt, _stream()))
+    check(lib.mi355_conv_state_update(state.data_ptr(), x.data_ptr(), _cols(x, "x", C), *args, S, C, taps, dt,
+                                      _stream()))
+    return out
+
+
+def gated_delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, beta: torch.Tensor, decay: torch.Tensor,
+                     a_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
+                     positions: torch.Tensor, state_slots: torch.Tensor, num_heads: int, num_kv_heads: int,
+                     head_dim: int, v_dim: int, per_channel: bool = False, out: torch.Tensor | None = None):
+    """The gated delta rule over packed chunks.  qkv [tokens, C] holds q (kv_heads x head_dim) at column
+    q_off, k at k_off, v (heads x v_dim) at v_off; beta [tokens, heads] and decay [tokens, heads] or
+    [tokens, heads * head_dim] are raw projection outputs (column slices are fine); a_log [heads] and
+    dt_bias (decay's width) float32; state float32 [slots, heads, head_dim, v_dim].
+    Returns o float32 [tokens, heads, v_dim]."""
+    dt = _dt3(qkv, "qkv")
+    T = qkv.shape[0]
+    S = cu_seqlens.numel() - 1
+    width = num_heads * head_dim if per_channel else num_heads
+    if tuple(state.shape[1:]) != (num_heads, head_dim, v_dim):
+        raise ValueError("state must be [slots, heads, head_dim, v_dim]")
+    need = max(q_off + num_kv_heads * head_dim, k_off + num_kv_heads * head_dim, v_off + num_heads * v_dim)
+    if qkv.dim() != 2 or qkv.shape[1] < need or not qkv.is_contiguous():
+        raise ValueError("qkv must be contiguous [tokens, >= the q / k / v columns]")
+    if out is None:
+        out = torch.empty(T, num_heads, v_dim, dtype=torch.float32, device=qkv.device)
+    check(lib.mi355_gated_delta_rule(
+        _f32(out, "out", T * num_heads * v_dim), qkv.data_ptr(), qkv.shape[1], q_off, k_off, v_off,
+        _same(beta, qkv, "beta"), _cols(beta, "beta", num_heads), _same(decay, qkv, "decay"), _cols(decay, "decay", width),
+        _f32(a_log, "a_log", num_heads), _f32(dt_bias, "dt_bias", width), int(per_channel), _f32(state, "state"),
+        _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(positions, "positions", torch.int64, T),
+        _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, num_kv_heads, head_dim, v_dim, dt, _stream()))
+    return out
