@@ -740,7 +740,7 @@ int32_t mi355_allreduce_oneshot_destroy(void* comm);
  * keeps the residual in the model's 16-bit type).  `dtype` is the storage type of activations and
  * weights: MI355_BF16, MI355_F16 or MI355_F32; sums, means and transcendentals are fp32 always.
  *   embed_scale_f32       resid[t] = embed[ids[t]] * scale
- *   resid_add_f32         resid[t] += other[t] (fp32, may be null) + vec (one row, may be null)
+ *   resid_add_f32         resid[t] += other[t] (fp32) + rows[t] (dtype) + vec (one row, dtype); each may be null
  *   add_rms_norm_f32      resid += add (may be null); out = resid / sqrt(mean(resid^2) + eps) * w,
  *                         w one number (weight_numel 1) or one per column (weight_numel == width)
  *   rms_norm_mix_f32      resid += alpha * (rmsnorm(xa) * wa + rmsnorm(xb) * wb); xb / wb may be null
@@ -751,8 +751,8 @@ int32_t mi355_allreduce_oneshot_destroy(void* comm);
  */
 int32_t mi355_embed_scale_f32(float* out, const void* embed, const int64_t* ids, int64_t num_tokens,
                               int32_t width, int64_t vocab, float scale, int32_t dtype, void* stream);
-int32_t mi355_resid_add_f32(float* resid, const float* other, const void* vec, int64_t num_tokens,
-                            int32_t width, int32_t dtype, void* stream);
+int32_t mi355_resid_add_f32(float* resid, const float* other, const void* rows, const void* vec,
+                            int64_t num_tokens, int32_t width, int32_t dtype, void* stream);
 int32_t mi355_add_rms_norm_f32(void* out, float* resid, const void* add, const void* weight,
                                int32_t weight_numel, int64_t num_tokens, int32_t width, float eps,
                                int32_t dtype, void* stream);

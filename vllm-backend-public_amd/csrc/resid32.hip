@@ -1,6 +1,6 @@
 // Pointwise and normalisation kernels for decoders that keep the residual stream in fp32:
 //   embed_scale_f32          resid = embed[id] * scale
-//   resid_add_f32            resid += other (fp32 rows) + vec (one row, broadcast)
+//   resid_add_f32            resid += other (fp32 rows) + rows (activation rows) + vec (one row, broadcast)
 //   add_rms_norm_f32         resid += add; out = resid / rms(resid) * w      (w: one number or a vector)
 //   rms_norm_mix_f32         resid += alpha * (xa / rms(xa) * wa + xb / rms(xb) * wb)
 //   gelu_tanh_and_mul        out = gelu_tanh(gate) * up for rows holding gate | up
@@ -24,11 +24,13 @@ __global__ __launch_bounds__(256) void embed_scale_f32_kernel(float* __restrict_
 
 template <typename T>
 __global__ __launch_bounds__(256) void resid_add_f32_kernel(float* __restrict__ resid, const float* __restrict__ other,
+                                                            const typename Elem<T>::S* __restrict__ rows,
                                                             const typename Elem<T>::S* __restrict__ vec, int W) {
   const int64_t t = blockIdx.x;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float v = MI355_LD(float, resid, resid + t * W + c);
     if (other != nullptr) v += MI355_LD(float, other, other + t * W + c);
+    if (rows != nullptr) v += MI355_LDF(T, rows, rows + t * W + c);
     if (vec != nullptr) v += MI355_LDF(T, vec, vec + c);
     MI355_ST(float, resid, resid + t * W + c, v);
   }
@@ -168,15 +170,16 @@ extern "C" int32_t mi355_embed_scale_f32(float* out, const void* embed, const in
   return check_launch("embed_scale_f32");
 }
 
-extern "C" int32_t mi355_resid_add_f32(float* resid, const float* other, const void* vec, int64_t num_tokens,
+extern "C" int32_t mi355_resid_add_f32(float* resid, const float* other, const void* rows, const void* vec, int64_t num_tokens,
                                        int32_t width, int32_t dtype, void* stream) {
   MI355_REQUIRE(resid, MI355_ERR_INVALID, "resid_add_f32: null pointer");
   MI355_REQUIRE(num_tokens >= 0 && width > 0, MI355_ERR_INVALID, "resid_add_f32: sizes");
   REQ_DTYPE(dtype);
-  if (num_tokens == 0 || (!other && !vec)) return MI355_OK;
+  if (num_tokens == 0 || (!other && !rows && !vec)) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((resid_add_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s, resid,
-                                                  other, static_cast<const Elem<TT>::S*>(vec), width));
+                                                  other, static_cast<const Elem<TT>::S*>(rows),
+                                                  static_cast<const Elem<TT>::S*>(vec), width));
   return check_launch("resid_add_f32");
 }
 

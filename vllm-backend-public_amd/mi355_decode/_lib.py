@@ -97,7 +97,7 @@ def _load() -> ctypes.CDLL:
         "mi355_allreduce_oneshot_destroy": (I32, [P]),
         "mi355_linear_decode": (I32, [P, I64, P, I64, P, P, I32, I32, I32, I32, I32, P]),
         "mi355_embed_scale_f32": (I32, [P, P, P, I64, I32, I64, F, I32, P]),
-        "mi355_resid_add_f32": (I32, [P, P, P, I64, I32, I32, P]),
+        "mi355_resid_add_f32": (I32, [P, P, P, P, I64, I32, I32, P]),
         "mi355_add_rms_norm_f32": (I32, [P, P, P, P, I32, I64, I32, F, I32, P]),
         "mi355_rms_norm_mix_f32": (I32, [P, P, P, P, P, I64, I32, F, F, I32, P]),
         "mi355_gelu_tanh_and_mul": (I32, [P, P, I64, I64, I32, I32, P]),

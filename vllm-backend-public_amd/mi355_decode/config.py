@@ -14,7 +14,7 @@ import os
 from dataclasses import dataclass, field
 from typing import Any, Optional
 
-SUPPORTED_ARCHS = ("LlamaForCausalLM", "Qwen2ForCausalLM", "MistralForCausalLM", "OPTForCausalLM")
+SUPPORTED_ARCHS = ("LlamaForCausalLM", "Qwen2ForCausalLM", "MistralForCausalLM", "OPTForCausalLM", "Lozupel")
 
 # Well-known geometries, used when --model names one of them and no local
 # config.json exists (synthetic-weight benchmarking; there is no network).
@@ -48,6 +48,102 @@ def _known_key(name: str) -> Optional[str]:
 
 
 @dataclass
+class WindowAttnSpec:
+    """Sliding-window attention with sigmoid weights: sigmoid(q.k * scale * temp[h] + bias[h]) for the
+    keys j with 0 <= i - j < window, not normalised over keys; rotary positions on the first rot_dims
+    coordinates of each head; one output gate per head."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    window: int
+    rot_dims: int
+    rot_base: float
+    scale: float
+
+
+@dataclass
+class DeltaSpec:
+    """Gated delta rule mixer: heads value heads of vdim channels on kv_heads query / key heads of dim
+    channels, a causal convolution of `conv` taps on q, k and v.  per_channel: one decay per key
+    channel (projected through a low-rank pair, as is the output gate, which is then a sigmoid)
+    instead of one per head (full-rank projections, SiLU gate)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    per_channel: bool = False
+
+
+@dataclass
+class HybridLayerSpec:
+    kind: str                               # "delta": one DeltaSpec; "parallel": window attention beside a delta mixer
+    delta: DeltaSpec = None
+    attn: Optional[WindowAttnSpec] = None
+    ff: Optional[int] = None                # width of the gated feed-forward, None: the layer has none
+
+
+@dataclass
+class HybridSpec:
+    """A decoder whose layers each name their sequence mixer, with an optional weight-shared loop:
+    layers loop_start .. loop_stop - 1 run loop_times times in a row (separate cache and state per
+    pass); before every pass a learned vector is added to the residual, and before every pass but
+    the first the embedding output too."""
+    layers: list
+    embed_scale: float = 1.0
+    logit_softcap: Optional[float] = None
+    loop_start: int = 0
+    loop_stop: int = 0
+    loop_times: int = 0                     # 0: no loop
+
+    def runs(self):
+        """[(layer index, pass number or None)] in execution order: one cache / state each."""
+        n = len(self.layers)
+        if self.loop_times <= 0:
+            return [(i, None) for i in range(n)]
+        out = [(i, None) for i in range(self.loop_start)]
+        for t in range(self.loop_times):
+            out += [(i, t) for i in range(self.loop_start, self.loop_stop)]
+        return out + [(i, None) for i in range(self.loop_stop, n)]
+
+    @classmethod
+    def from_lozupel(cls, d: dict) -> "HybridSpec":
+        def delta(m, per_channel):
+            return DeltaSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                             vdim=int(m["vdim"]), conv=int(m["conv"]), per_channel=per_channel)
+        layers = []
+        for spec in d["layers"]:
+            m, mlp = spec["mixer"], spec.get("mlp")
+            if mlp is not None and mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"feed-forward kind {mlp.get('kind')!r} is not supported (dense)")
+            ff = int(mlp["ff"]) if mlp is not None else None
+            if spec["type"] == "delta":
+                layers.append(HybridLayerSpec("delta", delta=delta(m, False), ff=ff))
+            elif spec["type"] == "parallel":
+                a = m["left"]
+                attn = WindowAttnSpec(heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]),
+                                      vdim=int(a["vdim"]), window=int(a["mask"]["size"]),
+                                      rot_dims=int(a["rot"]["dims"]), rot_base=float(a["rot"]["base"]),
+                                      scale=float(a["scale"]))
+                layers.append(HybridLayerSpec("parallel", delta=delta(m["right"], True), attn=attn, ff=ff))
+            else:
+                raise ValueError(f"layer type {spec['type']!r} is not supported (delta, parallel)")
+        for L in layers:
+            for m in (L.delta, L.attn):
+                if m is not None and (m.heads % m.kv_heads or m.heads < 1):
+                    raise ValueError(f"kv_heads {m.kv_heads} must divide heads {m.heads}")
+        loop = d.get("loop") or {}
+        out = cls(layers=layers, embed_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
+                  logit_softcap=(float(d["logit_softcap"]) if d.get("logit_softcap") else None),
+                  loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
+                  loop_times=int(loop.get("times", 0)))
+        if out.loop_times > 0 and not 0 <= out.loop_start < out.loop_stop <= len(layers):
+            raise ValueError(f"loop {out.loop_start}..{out.loop_stop} does not fit {len(layers)} layers")
+        return out
+
+
+@dataclass
 class ModelConfig:
     architecture: str
     vocab_size: int
@@ -71,6 +167,21 @@ class ModelConfig:
     position_offset: int = 0
     # the type the checkpoint's weights are stored in (config.json's torch_dtype / dtype), if it says
     torch_dtype: Optional[str] = None
+    # family "hybrid": the per-layer mixers, loop and output constants; the Llama-shaped fields above
+    # then hold the width, the vocabulary and the largest head geometry for sizing only
+    hybrid: Optional[HybridSpec] = None
+
+    @classmethod
+    def _from_lozupel_dict(cls, d: dict) -> "ModelConfig":
+        spec = HybridSpec.from_lozupel(d)
+        mixers = [m for L in spec.layers for m in (L.attn, L.delta) if m is not None]
+        return cls(architecture="Lozupel", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]),
+                   intermediate_size=max([L.ff or 0 for L in spec.layers] + [0]), num_hidden_layers=len(spec.layers),
+                   num_attention_heads=max(m.heads for m in mixers), num_key_value_heads=max(m.kv_heads for m in mixers),
+                   head_dim=max(m.dim for m in mixers), rope_theta=0.0, rope_scaling=None,
+                   rms_norm_eps=float(d["norm"]["eps"]), max_position_embeddings=int(d.get("max_positions", 1 << 17)),
+                   tie_word_embeddings=False, attention_bias=False, bos_token_id=d.get("bos_token_id"),
+                   eos_token_id=d.get("eos_token_id"), family="hybrid", hybrid=spec)
 
     @classmethod
     def _from_opt_dict(cls, d: dict) -> "ModelConfig":
@@ -96,7 +207,7 @@ class ModelConfig:
 
     @classmethod
     def from_dict(cls, d: dict) -> "ModelConfig":
-        archs = d.get("architectures") or ["LlamaForCausalLM"]
+        archs = d.get("architectures") or ([d["architecture"]] if d.get("architecture") else ["LlamaForCausalLM"])
         arch = archs[0]
         if arch not in SUPPORTED_ARCHS:
             raise ValueError(f"architecture {arch!r} is not supported (supported: {SUPPORTED_ARCHS})")
@@ -105,6 +216,10 @@ class ModelConfig:
         if arch == "OPTForCausalLM":
             cfg = cls._from_opt_dict(d)
             cfg.torch_dtype = stored
+            return cfg
+        if arch == "Lozupel":
+            cfg = cls._from_lozupel_dict(d)
+            cfg.torch_dtype = stored or "bfloat16"
             return cfg
         nh = d["num_attention_heads"]
         rope_params = d.get("rope_parameters") or {}
@@ -205,6 +320,7 @@ class EngineArgs:
     trust_remote_code: bool = False
     device: str = "auto"
     num_layers_override: Optional[int] = None      # testing / bounded benchmarks only
+    num_gpu_blocks_override: Optional[int] = None  # KV pages to allocate instead of what the memory budget gives
     extra: dict = field(default_factory=dict)      # accepted-and-ignored engine flags
 
     def resolved_dtype(self, checkpoint_dtype: Optional[str] = None) -> str:
@@ -235,4 +351,6 @@ class EngineArgs:
             raise ValueError(f"--quantization {self.quantization!r} is not supported (fp8 or none)")
         if self.max_num_seqs < 1:
             raise ValueError("--max-num-seqs must be >= 1")
+        if self.num_gpu_blocks_override is not None and self.num_gpu_blocks_override < 1:
+            raise ValueError("--num-gpu-blocks-override must be >= 1")
         self.resolved_dtype()

@@ -56,6 +56,27 @@ class BlockAllocator:
         self._free.extend(reversed(blocks))
 
 
+class SlotAllocator:
+    """Free list of per-sequence state slots (recurrent and convolution state of models whose
+    mixers carry one): a sequence holds one slot from admission to release."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def allocate(self) -> int:
+        if not self._free:
+            raise NoFreeBlocks("no free state slot")
+        return self._free.pop()
+
+    def free(self, slot: int) -> None:
+        self._free.append(slot)
+
+
 @dataclass(eq=False)          # identity semantics: sequences live in scheduler lists
 class Sequence:
     request_id: str
@@ -64,6 +85,7 @@ class Sequence:
     arrival_time: float = field(default_factory=time.perf_counter)
     output_ids: List[int] = field(default_factory=list)
     blocks: List[int] = field(default_factory=list)
+    state_slot: Optional[int] = None # recurrent-state slot (models that carry state), held while running
     num_computed: int = 0            # tokens whose K/V are in the cache
     first_token_time: Optional[float] = None
     finish_time: Optional[float] = None
@@ -109,8 +131,9 @@ class RequestOutput:
 
 class Scheduler:
     def __init__(self, allocator: BlockAllocator, max_num_seqs: int, max_num_batched_tokens: int,
-                 max_model_len: int):
+                 max_model_len: int, slots: Optional[SlotAllocator] = None):
         self.alloc = allocator
+        self.slots = slots                       # None: the model carries no per-sequence state
         self.max_num_seqs = max_num_seqs
         self.max_tokens = max_num_batched_tokens
         self.max_model_len = max_model_len
@@ -136,6 +159,26 @@ class Scheduler:
             self.running.remove(seq)
         self.alloc.free(seq.blocks)
         seq.blocks = []
+        if seq.state_slot is not None:
+            self.slots.free(seq.state_slot)
+            seq.state_slot = None
+
+    def admit(self, seq: Sequence, n_tokens: int) -> None:
+        """Pages for n_tokens tokens and (models with state) a state slot; the sequence runs from now on.
+        A sequence that starts at position 0 finds its slot's state reset by the first step that runs it."""
+        if self.slots is not None and seq.state_slot is None:
+            if self.slots.num_free == 0:
+                raise NoFreeBlocks("no free state slot")
+            seq.state_slot = self.slots.allocate()
+        try:
+            self._grow(seq, n_tokens)
+        except NoFreeBlocks:
+            if seq.state_slot is not None and seq not in self.running:
+                self.slots.free(seq.state_slot)
+                seq.state_slot = None
+            raise
+        if seq not in self.running:
+            self.running.append(seq)
 
     @staticmethod
     def prefill_target(seq: Sequence) -> int:
@@ -181,9 +224,10 @@ class Scheduler:
             # a sequence is admitted only if all its tokens fit in the pool right now
             if self._blocks_for(seq.total_len + 1) > self.alloc.num_free:
                 break
+            if self.slots is not None and self.slots.num_free == 0:
+                break
             self.waiting.popleft()
-            self._grow(seq, seq.total_len + 1)
-            self.running.append(seq)
+            self.admit(seq, seq.total_len + 1)
             n = min(self.prefill_target(seq), budget)
             chunks.append((seq, 0, n))
             budget -= n
@@ -218,7 +262,10 @@ class LLMEngine:
         self.device = runner.device
         self.max_model_len = max_model_len
         self.alloc = BlockAllocator(runner.num_blocks)
-        self.sched = Scheduler(self.alloc, max_num_seqs, max_num_batched_tokens, max_model_len)
+        # models whose mixers carry per-sequence state (recurrences, convolutions) keep it in slots
+        n_slots = int(getattr(runner, "num_state_slots", 0))
+        self.slots = SlotAllocator(n_slots) if n_slots > 0 else None
+        self.sched = Scheduler(self.alloc, max_num_seqs, max_num_batched_tokens, max_model_len, slots=self.slots)
         self.eos = set(eos_token_ids or [])
         self.seqs: Dict[str, Sequence] = {}
         # host mirrors (numpy views of pinned memory) of the runner's packed decode inputs,
@@ -308,7 +355,10 @@ class LLMEngine:
         """Top-k width a step has to compute: the largest any of its requests asked for; -1: none did."""
         return max([s.params.logprobs for s in seqs if s.params.logprobs is not None], default=-1)
 
-    def _prefill(self, chunks) -> List[RequestOutput]:
+    def _stage_chunks(self, chunks):
+        """Packed inputs of one step over chunks [(seq, first position, tokens)]: token ids, positions,
+        cache slots, block tables, row offsets, context lengths; plus the runner keywords a model
+        with per-sequence state needs."""
         MB = self.runner.max_blocks
         toks, pos, slots, cu, ctx = [], [], [], [0], []
         bt = np.zeros((len(chunks), MB), dtype=np.int32)
@@ -322,8 +372,18 @@ class LLMEngine:
             cu.append(cu[-1] + n)
             ctx.append(start + n)
             bt[i, : len(seq.blocks)] = seq.blocks
+        kw = {}
+        if self.slots is not None:
+            kw["state_slots"] = np.asarray([c[0].state_slot for c in chunks], dtype=np.int32)
+        args = (np.concatenate(toks), np.concatenate(pos), np.concatenate(slots), bt, np.asarray(cu, dtype=np.int32),
+                np.asarray(ctx, dtype=np.int32), max(n for _, _, n in chunks))
+        return args, cu, kw
+
+    def _prefill(self, chunks) -> List[RequestOutput]:
+        args, cu, kw = self._stage_chunks(chunks)
         k = self._logprobs_k([c[0] for c in chunks])
-        kw = {"logprobs": k} if k >= 0 else {}
+        if k >= 0:
+            kw["logprobs"] = k
         # prompt scoring: row r of the packed batch predicts the prompt token after it
         rows, targets, owners = [], [], []
         for i, (seq, start, n) in enumerate(chunks):
@@ -340,10 +400,7 @@ class LLMEngine:
         if rows:
             kw["prompt_logprobs"] = (max(c[0].params.prompt_logprobs or 0 for c in chunks),
                                      np.asarray(rows, dtype=np.int64), np.asarray(targets, dtype=np.int64))
-        nxt = self.runner.run_prefill(np.concatenate(toks), np.concatenate(pos), np.concatenate(slots), bt,
-                                      np.asarray(cu, dtype=np.int32), np.asarray(ctx, dtype=np.int32),
-                                      max(n for _, _, n in chunks),
-                                      sampling=self._sampling_arrays([c[0] for c in chunks]), **kw)
+        nxt = self.runner.run_prefill(*args, sampling=self._sampling_arrays([c[0] for c in chunks]), **kw)
         if rows:                                     # (the usual result, one (logprob, top) per scored row)
             nxt, plps = nxt
             for seq, (lp, top) in zip(owners, plps):
@@ -379,7 +436,11 @@ class LLMEngine:
         n64, n32 = self._hosts[st]
         n64[2 * B:] = -1                      # neutral padding: store nothing,
         n32[:B] = 0                           # attend to nothing
-        bt = n32[B:].reshape(B, MB)
+        bt = n32[B:B + B * MB].reshape(B, MB)
+        if self.slots is not None:
+            n32[B + B * MB:] = self.slots.num_slots   # padding rows write their state to the spare slot
+            for i, seq in enumerate(seqs):
+                n32[B + B * MB + i] = seq.state_slot
         for i, seq in enumerate(seqs):
             p = seq.total_len - 1 + seq.inflight   # position of the newest token (not yet in the cache)
             if not ahead:
@@ -431,6 +492,51 @@ class LLMEngine:
             self._append_token(seq, int(tok), now)
             outs.append(self._output(seq, [seq.output_ids[-1]], lps[i] if lps else None))
         return outs
+
+    # ------------------------------------------------------------------ #
+    # teacher-forced steps: the caller names every token (trace replay, scoring)
+    # ------------------------------------------------------------------ #
+    def forced_step(self, entries, end=()) -> np.ndarray:
+        """One step over given tokens instead of sampled ones.  entries: [(request id, [token ids],
+        [indices among these tokens whose logits are wanted])]; a request is admitted at its first
+        entry (pages and, for models with state, a slot), continues from its cache and state at later
+        ones, and may sit a step out.  All entries run as ONE batch through the same step function,
+        scheduler bookkeeping and cache as generation.  `end`: requests released after the step.
+        Returns the wanted logits, float32 [wanted, vocab], in the order of entries and indices."""
+        if self._pending:
+            raise RuntimeError("forced_step while decode steps are in flight")
+        chunks, rows, at = [], [], 0
+        for rid, toks, want in entries:
+            if not toks:
+                raise ValueError(f"request {rid}: no tokens in this step")
+            bad = [t for t in toks if not 0 <= t < self.runner.V]
+            if bad:
+                raise ValueError(f"token id {bad[0]} outside the vocabulary (size {self.runner.V})")
+            seq = self.seqs.get(rid)
+            if seq is None:
+                seq = Sequence(rid, [], SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True))
+                self.seqs[rid] = seq
+            start = seq.num_computed
+            if start + len(toks) > self.max_model_len:
+                raise ValueError(f"request {rid} grows past max_model_len {self.max_model_len}")
+            seq.prompt_ids.extend(int(t) for t in toks)
+            self.sched.admit(seq, start + len(toks))       # NoFreeBlocks: the pool is too small for the live requests
+            chunks.append((seq, start, len(toks)))
+            rows += [at + int(j) for j in want]
+            at += len(toks)
+        logits = np.zeros((0, self.runner.V), dtype=np.float32)
+        if chunks:
+            args, _, kw = self._stage_chunks(chunks)
+            logits = self.runner.run_prefill(*args, logit_rows=np.asarray(rows, dtype=np.int64), **kw)
+            self.stats["prefill_steps"] += 1
+            for seq, start, n in chunks:
+                seq.num_computed = start + n
+                self.stats["prefill_tokens"] += n
+        for rid in end:
+            seq = self.seqs.pop(rid, None)
+            if seq is not None:
+                self.sched.release(seq)
+        return logits
 
     def step(self) -> List[RequestOutput]:
         if not self._pending:

@@ -58,6 +58,7 @@ def make_arg_parser() -> argparse.ArgumentParser:
     p.add_argument("--max-num-seqs", type=int, default=256)
     p.add_argument("--max-num-batched-tokens", type=int, default=8192)
     p.add_argument("--block-size", type=int, default=16)
+    p.add_argument("--num-gpu-blocks-override", type=int, default=None)
     p.add_argument("--gpu-memory-utilization", type=float, default=0.9)
     p.add_argument("--tensor-parallel-size", "-tp", type=int, default=1)
     p.add_argument("--pipeline-parallel-size", "-pp", type=int, default=1)
@@ -109,7 +110,7 @@ def parse_args(argv: Optional[List[str]] = None) -> Tuple[argparse.Namespace, En
         gpu_memory_utilization=ns.gpu_memory_utilization, tensor_parallel_size=ns.tensor_parallel_size,
         pipeline_parallel_size=ns.pipeline_parallel_size, quantization=quant, load_format=ns.load_format,
         seed=ns.seed, enforce_eager=os.environ.get("MI355_ENFORCE_EAGER") == "1",
-        trust_remote_code=ns.trust_remote_code,
+        trust_remote_code=ns.trust_remote_code, num_gpu_blocks_override=ns.num_gpu_blocks_override,
         device=extra.get("device", "auto") or "auto", extra=extra)
     args.validate()
     return ns, args

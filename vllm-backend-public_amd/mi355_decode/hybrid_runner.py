@@ -1,0 +1,314 @@
+"""One model step on one GPU for hybrid decoders (config.HybridSpec; the Lozupel design): every
+layer names its sequence mixer -- a gated delta rule (a linear recurrence with a matrix state per
+head), or a sliding-window attention with sigmoid weights beside such a recurrence -- and may carry a
+gated feed-forward; a span of layers can run several times with shared weights.
+
+What differs from ModelRunner's decoders, and where it lives:
+  * the residual stream is float32 (csrc/resid32.hip: norms with one learned number or a vector,
+    residual adds, the gelu-tanh gate, the logit soft cap); activations and weights are bfloat16
+    (or float32 throughout with dtype float32: every kernel here is built for both);
+  * K/V pages hold rotated keys [blocks, kv_heads, 16, dim] and values [blocks, kv_heads, 16, vdim],
+    one pair per layer RUN (a looped layer has one per pass), on the engine's block tables;
+  * recurrent and convolution state lives in per-sequence slots (engine.SlotAllocator), again one
+    set per layer run; a chunk that starts at position 0 resets its slot;
+  * one step function, `_forward`, serves prompts, portions of prompts and decoded tokens in one
+    packed batch (csrc/seqmix.hip).  run_prefill drives it eagerly; the decode step drives the same
+    function from the static step inputs and is captured into a HIP graph per batch bucket.
+
+Shares ModelRunner's step machinery: static step inputs and pinned staging, graph capture and
+replay, run-ahead, sampling, log-probabilities.  One GPU only.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import numpy as np
+import torch
+
+from . import ops
+from ._lib import BLOCK_SIZE
+from .config import ModelConfig
+from .model_runner import ModelRunner, batch_buckets
+from .weights import ModelWeights
+
+
+def rotary_table(rot_dims: int, base: float, max_pos: int, device) -> torch.Tensor:
+    """float32 [max_pos, rot_dims] = cos | sin of pos * base^(-2i / rot_dims), i < rot_dims / 2."""
+    half = rot_dims // 2
+    inv = float(base) ** (-2.0 * torch.arange(half, dtype=torch.float32, device=device) / rot_dims)
+    ang = torch.arange(max_pos, dtype=torch.float32, device=device)[:, None] * inv[None, :]
+    return torch.cat([ang.cos(), ang.sin()], dim=1).contiguous()
+
+
+class StepBatch:
+    """Device-side description of one packed step (see csrc/seqmix.hip)."""
+    __slots__ = ("ids", "positions", "slot_mapping", "block_tables", "cu_seqlens", "tok_seq", "state_slots",
+                 "num_tokens", "num_seqs")
+
+    def __init__(self, ids, positions, slot_mapping, block_tables, cu_seqlens, tok_seq, state_slots):
+        self.ids, self.positions, self.slot_mapping, self.block_tables = ids, positions, slot_mapping, block_tables
+        self.cu_seqlens, self.tok_seq, self.state_slots = cu_seqlens, tok_seq, state_slots
+        self.num_tokens, self.num_seqs = int(ids.numel()), int(cu_seqlens.numel()) - 1
+
+
+class WindowAttention:
+    """Sliding-window attention with sigmoid weights over the paged K/V of one layer run."""
+
+    def __init__(self, spec, lw, runner, cache_index: int):
+        self.s, self.lw, self.r, self.ci = spec, lw, runner, cache_index
+
+    def __call__(self, proj: torch.Tensor, b: StepBatch) -> torch.Tensor:
+        s, seg, r = self.s, self.lw.seg, self.r
+        q = proj[:, seg["lq"][0]: seg["lq"][0] + seg["lq"][1]]
+        k = proj[:, seg["lk"][0]: seg["lk"][0] + seg["lk"][1]]
+        v = proj[:, seg["lv"][0]: seg["lv"][0] + seg["lv"][1]]
+        g = proj[:, seg["lg"][0]: seg["lg"][0] + seg["lg"][1]]
+        kc, vc = r.k_cache[self.ci], r.v_cache[self.ci]
+        ops.rope_partial_kv_write(q, k, v, r.rotary(s.rot_dims, s.rot_base), b.positions, b.slot_mapping, kc, vc,
+                                  s.heads, s.kv_heads, s.dim, s.vdim)
+        o = ops.sigmoid_window_attn(q, kc, vc, b.block_tables, b.tok_seq, b.positions, self.lw.attn_temp,
+                                    self.lw.attn_bias, g, s.heads, s.window, s.scale)
+        return r.linear(o, self.lw.attn_o_w)
+
+
+class DeltaMixer:
+    """Gated delta rule with its convolution, decay, gate and output norm, on one layer run's state slots."""
+
+    def __init__(self, spec, lw, runner, state_index: int):
+        self.s, self.lw, self.r, self.si = spec, lw, runner, state_index
+
+    def __call__(self, proj: torch.Tensor, b: StepBatch) -> torch.Tensor:
+        s, lw, seg, r = self.s, self.lw, self.lw.seg, self.r
+        qk, vv = s.kv_heads * s.dim, s.heads * s.vdim
+        q0 = seg["q"][0]
+        if seg["k"][0] != q0 + qk or seg["v"][0] != q0 + 2 * qk:
+            raise RuntimeError("q | k | v of a delta mixer must be adjacent in the input projection")
+        conv_state, rec_state = r.conv_state[self.si], r.rec_state[self.si]
+        y = ops.causal_conv_silu(proj[:, q0: q0 + 2 * qk + vv], lw.conv_w, conv_state, b.tok_seq, b.positions,
+                                 b.cu_seqlens, b.state_slots)
+        beta = proj[:, seg["b"][0]: seg["b"][0] + s.heads]
+        if s.per_channel:
+            decay = r.linear(proj[:, seg["a1"][0]: seg["a1"][0] + seg["a1"][1]], lw.a2_w)
+            gate = r.linear(proj[:, seg["g1"][0]: seg["g1"][0] + seg["g1"][1]], lw.g2_w)
+        else:
+            decay = proj[:, seg["a"][0]: seg["a"][0] + s.heads]
+            gate = proj[:, seg["g"][0]: seg["g"][0] + vv]
+        o = ops.gated_delta_rule(y, 0, qk, 2 * qk, beta, decay, lw.a_log, lw.dt_bias, rec_state, b.cu_seqlens,
+                                 b.positions, b.state_slots, s.heads, s.kv_heads, s.dim, s.vdim,
+                                 per_channel=s.per_channel)
+        on = ops.gated_head_rms_norm(o, gate, lw.head_norm, r.eps, ops.ACT_SIGMOID if s.per_channel else ops.ACT_SILU)
+        return r.linear(on, lw.delta_o_w)
+
+
+class HybridRunner(ModelRunner):
+    def __init__(self, cfg: ModelConfig, weights: ModelWeights, dtype: torch.dtype, device, num_blocks: int,
+                 max_num_seqs: int, max_model_len: int, tp_rank: int = 0, tp_size: int = 1, tp_group=None,
+                 use_graphs: bool = True, decode_splits: Optional[int] = None, tiled_linears: Optional[bool] = None,
+                 weight_fp8: bool = False, num_state_slots: Optional[int] = None):
+        if cfg.family != "hybrid" or cfg.hybrid is None:
+            raise ValueError("HybridRunner runs hybrid decoders")
+        if tp_size != 1:
+            raise ValueError("hybrid decoders run on one GPU (tensor_parallel_size 1)")
+        if weight_fp8:
+            raise ValueError("--quantization fp8 is not available for hybrid decoders")
+        if dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            raise ValueError(f"dtype {dtype} not supported")
+        self.cfg, self.w, self.dtype, self.device = cfg, weights, dtype, torch.device(device)
+        self.spec = spec = cfg.hybrid
+        self.tp_rank, self.tp_size, self.tp_group = 0, 1, None
+        self.H, self.V, self.Vl = cfg.hidden_size, cfg.vocab_size, cfg.vocab_size
+        self.vocab_sharded, self.vocab_offset = False, 0
+        self.eps = cfg.rms_norm_eps
+        self.L = len(spec.layers)
+        self.num_blocks, self.max_num_seqs, self.max_model_len = int(num_blocks), int(max_num_seqs), int(max_model_len)
+        self.max_blocks = (self.max_model_len + BLOCK_SIZE - 1) // BLOCK_SIZE
+        self.use_graphs = use_graphs
+        self.allow_eager_fallback = False
+        self.capture_failures = self.tune_failures = 0
+        self.oneshot = None
+        self.oneshot_calls = self.fused_allreduce_norms = self.oneshot_key_reductions = self.oneshot_fallbacks = 0
+        self._no_collectives = False
+        self.decode_splits = decode_splits
+        self.weight_fp8 = self.single_weight_copy = False
+        self.tiled, self.tiled_policy, self._modes, self.tiled_shapes = None, "off", {}, {}
+        # one spare slot past the engine's: padding rows of a decode graph park their state there
+        self.num_state_slots = int(num_state_slots if num_state_slots is not None else max_num_seqs)
+        dev = self.device
+        self._rotary = {}
+        # caches and state, one set per layer RUN (a looped layer: one per pass)
+        self.runs = spec.runs()
+        self.k_cache, self.v_cache, self.conv_state, self.rec_state, self.mixers = [], [], [], [], []
+        for li, _ in self.runs:
+            L, lw = spec.layers[li], weights.layers[li]
+            D = L.delta
+            attn = None
+            if L.attn is not None:
+                A = L.attn
+                self.k_cache.append(torch.zeros(self.num_blocks, A.kv_heads, BLOCK_SIZE, A.dim, dtype=dtype, device=dev))
+                self.v_cache.append(torch.zeros(self.num_blocks, A.kv_heads, BLOCK_SIZE, A.vdim, dtype=dtype, device=dev))
+                attn = WindowAttention(A, lw, self, len(self.k_cache) - 1)
+            chans = 2 * D.kv_heads * D.dim + D.heads * D.vdim
+            self.conv_state.append(torch.zeros(self.num_state_slots + 1, max(D.conv - 1, 0), chans, dtype=torch.float32,
+                                               device=dev))
+            self.rec_state.append(torch.zeros(self.num_state_slots + 1, D.heads, D.dim, D.vdim, dtype=torch.float32,
+                                              device=dev))
+            self.mixers.append((attn, DeltaMixer(D, lw, self, len(self.rec_state) - 1)))
+        B = self.max_num_seqs
+        self._init_step_inputs(extra_i32=1)
+        self.row_extra.fill_(self.num_state_slots)
+        self.logits = torch.zeros(B, self.V, dtype=dtype, device=dev)
+        self.graphs = {}
+        self.buckets = batch_buckets(B)
+        self._init_step_staging()
+        # a decode step is B chunks of one row each
+        self._dec_cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
+        self._dec_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        self.layer_trace = None                       # a list: _forward appends the residual after every layer run
+
+    # ------------------------------------------------------------------ #
+    def rotary(self, rot_dims: int, base: float) -> torch.Tensor:
+        key = (rot_dims, base)
+        if key not in self._rotary:
+            self._rotary[key] = rotary_table(rot_dims, base, self.max_blocks * BLOCK_SIZE, self.device)
+        return self._rotary[key]
+
+    def kv_cache_bytes_per_block(self) -> int:
+        return sum(t[0].numel() * t.element_size() for t in self.k_cache + self.v_cache)
+
+    def state_bytes_per_slot(self) -> int:
+        return sum(t[0].numel() * t.element_size() for t in self.conv_state + self.rec_state)
+
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x @ w.T: the weight-streaming kernel for decode-sized row counts where its layout rules
+        hold, a library GEMM otherwise (prefill; float32; odd widths)."""
+        M, K = x.shape
+        N = w.shape[0]
+        if (x.dtype != torch.float32 and M <= ops.LINEAR_DECODE_MAX_M and K % 32 == 0 and N % 4 == 0
+                and x.stride(1) == 1 and (M == 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0):
+            return ops.linear_decode(x, w, None, out=out)
+        if out is None:
+            return torch.mm(x, w.t())
+        return torch.mm(x, w.t(), out=out)
+
+    def tune(self, bucket: int) -> dict:
+        self._modes.setdefault(bucket, {})
+        return self._modes[bucket]
+
+    def warm_up(self) -> None:
+        return None
+
+    def capture(self, bucket: int) -> None:
+        """As ModelRunner.capture; the warm-up and capture runs park every row's state in the spare
+        slot, so that they cannot touch the state of live sequences."""
+        if bucket in self.graphs:
+            return
+        saved = self.row_extra.clone()
+        self.row_extra.fill_(self.num_state_slots)
+        try:
+            super().capture(bucket)
+        finally:
+            self.row_extra.copy_(saved)
+
+    def _use_tiled(self, b: int) -> bool:
+        return False
+
+    # ------------------------------------------------------------------ #
+    def _forward(self, b: StepBatch) -> torch.Tensor:
+        """All layers over one packed batch; returns the float32 residual stream [tokens, width]."""
+        w, spec = self.w, self.spec
+        resid = ops.embed_scale_f32(w.embed, b.ids, spec.embed_scale)
+        x0 = resid.clone() if spec.loop_times > 1 else None
+        pending = None                                 # a sub-layer output not yet added to the residual
+        last = len(self.runs) - 1
+        for ri, (li, t) in enumerate(self.runs):
+            L, lw = spec.layers[li], w.layers[li]
+            if t is not None and li == spec.loop_start:    # a pass begins: + embedding output (not the first) + its step vector
+                ops.resid_add_f32(resid, other=x0 if t > 0 else None, rows=pending, vec=w.loop_step[t])
+                pending = None
+            h = ops.add_rms_norm_f32(resid, lw.norm1, self.eps, add=pending)    # the add rides in the norm's launch
+            pending = None
+            proj = self.linear(h, lw.in_w)
+            attn, delta = self.mixers[ri]
+            if attn is not None:
+                ops.rms_norm_mix_f32(resid, attn(proj, b), lw.attn_out_norm, delta(proj, b), lw.delta_out_norm,
+                                     self.eps, 0.5)
+            else:
+                pending = delta(proj, b)
+            if L.ff:
+                h = ops.add_rms_norm_f32(resid, lw.norm2, self.eps, add=pending)
+                pending = self.linear(ops.gelu_tanh_and_mul(self.linear(h, lw.gate_up_w)), lw.down_w)
+            if pending is not None and (ri == last or self.layer_trace is not None):
+                ops.resid_add_f32(resid, rows=pending)
+                pending = None
+            if self.layer_trace is not None:
+                self.layer_trace.append(resid.clone())
+        return resid
+
+    def _logits(self, resid: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Final norm, head and soft cap over the given residual rows."""
+        h = ops.add_rms_norm_f32(resid, self.w.final_norm, self.eps)
+        z = self.linear(h, self.w.lm_head, out=out)
+        if self.spec.logit_softcap:
+            ops.softcap(z, self.spec.logit_softcap)
+        return z
+
+    # ------------------------------------------------------------------ #
+    def _decode_body(self, b: int) -> None:
+        batch = StepBatch(self.ids[:b], self.positions[:b], self.slots[:b], self.block_tables[:b],
+                          self._dec_cu[:b + 1], self._dec_seq[:b], self.row_extra[:b])
+        resid = self._forward(batch)
+        self._logits(resid, out=self.logits[:b])
+        self.greedy(self.logits[:b], self.next_ids[:b], ids_out=self.ids[:b])
+
+    def lm_head_logits(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        self.linear(x, self.w.lm_head, out=out)
+
+    def run_prefill(self, token_ids, positions, slot_mapping, block_tables, cu_seqlens, context_lens, max_q_len: int,
+                    sampling: Optional[dict] = None, logprobs: int = -1, prompt_logprobs=None, state_slots=None,
+                    logit_rows=None):
+        """As ModelRunner.run_prefill, over chunks that may be whole prompts, portions or single
+        tokens.  `state_slots`: the state slot of every chunk.  `logit_rows` (packed row numbers):
+        return float32 logits [rows, vocab] of those rows instead of sampling."""
+        if state_slots is None:
+            raise ValueError("hybrid decoders need the state slot of every chunk")
+        self._step_state_slots = np.asarray(state_slots, dtype=np.int32)
+        if logit_rows is None:
+            return super().run_prefill(token_ids, positions, slot_mapping, block_tables, cu_seqlens, context_lens,
+                                       max_q_len, sampling=sampling, logprobs=logprobs, prompt_logprobs=prompt_logprobs)
+        dev = self.device
+        t = lambda a, dt: torch.from_numpy(np.ascontiguousarray(a)).to(dev, dtype=dt, non_blocking=True)  # noqa: E731
+        resid = self._run_chunks(t(token_ids, torch.int64), t(positions, torch.int64), t(slot_mapping, torch.int64),
+                                 t(block_tables, torch.int32), t(cu_seqlens, torch.int32))
+        rows = np.asarray(logit_rows, dtype=np.int64)
+        if rows.size == 0:
+            torch.cuda.current_stream().synchronize()
+            return np.zeros((0, self.V), dtype=np.float32)
+        z = self._logits(resid.index_select(0, t(rows, torch.int64)))
+        return z.float().cpu().numpy()
+
+    def _run_chunks(self, token_ids, positions, slot_mapping, block_tables, cu_seqlens) -> torch.Tensor:
+        S = cu_seqlens.numel() - 1
+        lens = (cu_seqlens[1:] - cu_seqlens[:-1]).to(torch.int64)
+        tok_seq = torch.repeat_interleave(torch.arange(S, dtype=torch.int32, device=self.device), lens,
+                                          output_size=int(token_ids.numel()))
+        slots = torch.from_numpy(self._step_state_slots).to(self.device, non_blocking=True)
+        return self._forward(StepBatch(token_ids, positions, slot_mapping, block_tables.contiguous(), cu_seqlens,
+                                       tok_seq, slots))
+
+    def prefill(self, token_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor,
+                block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,
+                max_q_len: int, want_logits: bool = True, score=None):
+        """As ModelRunner.prefill: packed prompts (or prompt chunks), eager."""
+        resid = self._run_chunks(token_ids, positions, slot_mapping, block_tables, cu_seqlens)
+        if score is not None:
+            k, srows, targets = score
+            parts = []
+            for a in range(0, srows.numel(), 1024):
+                lg = self._logits(resid.index_select(0, srows[a:a + 1024]))
+                parts.append(self._logprobs(lg, targets[a:a + 1024], k))
+            self.prompt_scores = torch.cat(parts, dim=0)
+        rows = (cu_seqlens[1:] - 1).to(torch.int64)
+        logits = self._logits(resid.index_select(0, rows))
+        nxt = torch.empty(logits.shape[0], dtype=torch.int64, device=self.device)
+        self.greedy(logits, nxt)
+        return nxt, (logits if want_logits else None)

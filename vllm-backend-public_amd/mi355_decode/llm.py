@@ -18,7 +18,7 @@ from . import weights as W
 
 log = logging.getLogger("mi355_decode")
 
-TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float16": torch.float16}
+TORCH_DTYPE = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32}
 
 
 def init_distributed(tp_size: int):
@@ -60,6 +60,9 @@ def plan_num_blocks(args: EngineArgs, cfg: ModelConfig, tp_size: int, num_layers
     default utilisation is 0.0 (benchmark-vllm/models.py:8): then only the cap by
     free memory applies."""
     per_block = 2 * num_layers * (cfg.num_key_value_heads // tp_size) * BLOCK_SIZE * cfg.head_dim * elem_size
+    if cfg.family == "hybrid":                        # K and V pages of every layer run that has an attention
+        attn = [cfg.hybrid.layers[i].attn for i, _ in cfg.hybrid.runs() if cfg.hybrid.layers[i].attn is not None]
+        per_block = max(sum(a.kv_heads * (a.dim + a.vdim) for a in attn) * BLOCK_SIZE * elem_size, 1)
     blocks_per_seq = (max_model_len + BLOCK_SIZE - 1) // BLOCK_SIZE
     want = args.max_num_seqs * blocks_per_seq + 1
     free, total = torch.cuda.mem_get_info(device)
@@ -68,6 +71,10 @@ def plan_num_blocks(args: EngineArgs, cfg: ModelConfig, tp_size: int, num_layers
     budget = min(free - reserve, int(total * util) - (total - free) - reserve)
     fit = max(int(budget // per_block), 0)
     n = min(want, fit)
+    if args.num_gpu_blocks_override is not None:
+        if args.num_gpu_blocks_override > fit:
+            raise RuntimeError(f"--num-gpu-blocks-override {args.num_gpu_blocks_override}: only {fit} pages fit")
+        return int(args.num_gpu_blocks_override)
     if n < blocks_per_seq:
         raise RuntimeError(f"not enough GPU memory for the KV cache: {fit} pages fit, one sequence of "
                            f"max_model_len {max_model_len} needs {blocks_per_seq}")
@@ -80,7 +87,10 @@ def build_engine(args: EngineArgs, state_dict: Optional[dict] = None, model_conf
     rank, world, device, group = init_distributed(args.tensor_parallel_size)
     cfg = model_config or ModelConfig.from_pretrained(args.model)
     dtype = TORCH_DTYPE[args.resolved_dtype(cfg.torch_dtype)]
-    if (args.dtype or "").lower() in ("float32", "float"):
+    want32 = (args.dtype or "").lower() in ("float32", "float")
+    if want32 and cfg.family == "hybrid":
+        dtype = torch.float32                         # this family's kernels are built for 32-bit storage too
+    elif want32:
         log.warning("--dtype float32 requested: the gfx950 kernels compute in 16 bits, serving in %s (checkpoint "
                     "stored in %s)", args.resolved_dtype(cfg.torch_dtype), cfg.torch_dtype or "an unlabelled type")
     if args.block_size != BLOCK_SIZE:
@@ -110,7 +120,7 @@ def build_engine(args: EngineArgs, state_dict: Optional[dict] = None, model_conf
         weights = W.synthetic(cfg, dtype, device, seed=args.seed, **kw)
     # the runner keeps a second, fragment-tiled copy of the decode-time matrices
     fp8 = (args.quantization or "").lower() == "fp8"
-    if cfg.family == "opt":
+    if cfg.family in ("opt", "hybrid"):
         tiled_bytes = 0                               # its decode GEMMs stream the row-major weights
     else:
         tiled_bytes = sum(t.numel() * (1 if fp8 else t.element_size()) for lw in weights.layers
@@ -119,7 +129,7 @@ def build_engine(args: EngineArgs, state_dict: Optional[dict] = None, model_conf
     # MI355_SINGLE_WEIGHT_COPY=1: the tiled copy replaces the row-major one (half the weight memory:
     # what lets a model whose weights fill more than half the card be served at all); prefill then
     # rebuilds each layer's row-major matrices into scratch buffers, ~10 % more time to first token
-    single = os.environ.get("MI355_SINGLE_WEIGHT_COPY", "0") == "1" and cfg.family != "opt"
+    single = os.environ.get("MI355_SINGLE_WEIGHT_COPY", "0") == "1" and cfg.family not in ("opt", "hybrid")
     if single and weights.layers:
         lw0 = weights.layers[0]
         scratch = sum(t.numel() * t.element_size() for t in (lw0.qkv_w, lw0.gate_up_w, lw0.o_w, lw0.down_w))
@@ -132,6 +142,9 @@ def build_engine(args: EngineArgs, state_dict: Optional[dict] = None, model_conf
     if cfg.family == "opt":
         from .opt_runner import OPTRunner
         runner_cls = OPTRunner
+    elif cfg.family == "hybrid":
+        from .hybrid_runner import HybridRunner
+        runner_cls = HybridRunner
     extra = {"single_weight_copy": True} if single else {}
     runner = runner_cls(cfg, weights, dtype, device, num_blocks, args.max_num_seqs, max_model_len,
                          tp_rank=rank, tp_size=tp, tp_group=group, use_graphs=graphs,

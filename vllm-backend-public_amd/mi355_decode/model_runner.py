@@ -125,22 +125,9 @@ class ModelRunner:
         self.v_cache = [torch.zeros(self.num_blocks, self.nkv, self.d, BLOCK_SIZE, dtype=dtype, device=dev)
                         for _ in range(self.L)]
 
+        self._init_step_inputs()
         B = self.max_num_seqs
-        i64 = dict(dtype=torch.int64, device=dev)
-        i32 = dict(dtype=torch.int32, device=dev)
         f = dict(dtype=dtype, device=dev)
-        # step inputs (static addresses: the decode graphs read them).  Packed so the
-        # engine refreshes them with two host-to-device copies per step:
-        #   in64 = ids | positions | slots            (3 * B int64)
-        #   in32 = context_lens | block_tables        (B + B * max_blocks int32)
-        # one allocation (int32 words): the 64-bit part first, so that a step's inputs are ONE copy
-        self.inall = torch.zeros(6 * B + B + B * self.max_blocks, **i32)
-        self.in64 = self.inall[:6 * B].view(torch.int64)
-        self.in32 = self.inall[6 * B:]
-        self.ids, self.positions, self.slots = self.in64[:B], self.in64[B:2 * B], self.in64[2 * B:]
-        self.slots.fill_(-1)
-        self.ctx = self.in32[:B]
-        self.block_tables = self.in32[B:].view(B, self.max_blocks)
         # activations
         self.resid = torch.zeros(B, self.H, **f)
         self.x = torch.zeros(B, self.H, **f)
@@ -151,11 +138,6 @@ class ModelRunner:
         self.act = torch.zeros(B, self.F, **f)
         self.dn = torch.zeros(B, self.H, **f)
         self.logits = torch.zeros(B, self.Vl, **f)          # this rank's slice of the vocabulary
-        self.next_ids = torch.zeros(B, **i64)
-        self.keys = torch.zeros(B, **i64)             # argmax merge keys: zero between launches
-        # True while self.ids already holds the tokens the last decode step sampled (its argmax wrote
-        # them there too): a step launched ahead of the host then needs no copy of its input tokens
-        self._ids_synced = False
         self._max_splits = 16
         self.attn_ws = torch.empty(max(ops.decode_workspace_bytes(B, self.nh, self.d, self._max_splits), 16),
                                    dtype=torch.uint8, device=dev)
@@ -164,6 +146,38 @@ class ModelRunner:
         self._init_tiled(tiled_linears)
         if self.weight_fp8:
             self._fake_quantize_row_major()
+        self._init_step_staging()
+
+    def _init_step_inputs(self, extra_i32: int = 0) -> None:
+        """Static device buffers a decode step reads its inputs from (the decode graphs hold their
+        addresses).  `extra_i32`: int32 words per row appended after the block tables (models with
+        per-sequence state keep the row's state slot there)."""
+        dev = self.device
+        B = self.max_num_seqs
+        i64 = dict(dtype=torch.int64, device=dev)
+        i32 = dict(dtype=torch.int32, device=dev)
+        # step inputs (static addresses: the decode graphs read them).  Packed so the
+        # engine refreshes them with two host-to-device copies per step:
+        #   in64 = ids | positions | slots            (3 * B int64)
+        #   in32 = context_lens | block_tables        (B + B * max_blocks int32)
+        # one allocation (int32 words): the 64-bit part first, so that a step's inputs are ONE copy
+        self.inall = torch.zeros(6 * B + B + B * self.max_blocks + extra_i32 * B, **i32)
+        self.in64 = self.inall[:6 * B].view(torch.int64)
+        self.in32 = self.inall[6 * B:]
+        self.ids, self.positions, self.slots = self.in64[:B], self.in64[B:2 * B], self.in64[2 * B:]
+        self.slots.fill_(-1)
+        self.ctx = self.in32[:B]
+        self.block_tables = self.in32[B:B + B * self.max_blocks].view(B, self.max_blocks)
+        self.row_extra = self.in32[B + B * self.max_blocks:]
+        self.next_ids = torch.zeros(B, **i64)
+        self.keys = torch.zeros(B, **i64)             # argmax merge keys: zero between launches
+        # True while self.ids already holds the tokens the last decode step sampled (its argmax wrote
+        # them there too): a step launched ahead of the host then needs no copy of its input tokens
+        self._ids_synced = False
+
+    def _init_step_staging(self) -> None:
+        """Pinned host mirrors of the step inputs, results and sampling parameters."""
+        B = self.max_num_seqs
         # pinned host staging for the packed inputs and the sampled tokens: two sets, so
         # that the host can stage step n+1 while step n is still running
         self.h_alls = [torch.zeros(self.inall.numel(), dtype=torch.int32).pin_memory() for _ in range(self.NUM_STAGES)]

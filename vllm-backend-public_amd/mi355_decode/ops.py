@@ -964,16 +964,21 @@ def embed_scale_f32(embed: torch.Tensor, ids: torch.Tensor, scale: float, out: t
     return out
 
 
-def resid_add_f32(resid: torch.Tensor, other: torch.Tensor | None = None, vec: torch.Tensor | None = None):
-    """resid += other (float32 rows) + vec (one row of any supported dtype), in place."""
+def resid_add_f32(resid: torch.Tensor, other: torch.Tensor | None = None, rows: torch.Tensor | None = None,
+                  vec: torch.Tensor | None = None):
+    """resid (float32, in place) += other (float32 rows) + rows (activation rows) + vec (one row)."""
     T, W = resid.shape
-    dt = _DT[torch.float32]
-    if vec is not None:
-        dt = _dt3(vec, "vec")
-        if vec.numel() != W or not vec.is_contiguous():
-            raise ValueError("vec must be one contiguous row of the residual's width")
+    dt = None
+    for name, t, shape in (("rows", rows, (T, W)), ("vec", vec, (W,))):
+        if t is None:
+            continue
+        if (dt is not None and _DT[t.dtype] != dt) or t.numel() != T * W // (T if name == "vec" else 1) \
+                or not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous {shape}, rows and vec in one dtype")
+        dt = _dt3(t, name)
     check(lib.mi355_resid_add_f32(_f32(resid, "resid"), None if other is None else _f32(other, "other", T * W),
-                                  None if vec is None else vec.data_ptr(), T, W, dt, _stream()))
+                                  None if rows is None else rows.data_ptr(), None if vec is None else vec.data_ptr(),
+                                  T, W, _DT[torch.float32] if dt is None else dt, _stream()))
     return resid
 
 

@@ -68,6 +68,41 @@ class OPTLayerWeights:
 
 
 @dataclass
+class HybridLayerWeights:
+    """One layer of a hybrid decoder (config.HybridLayerSpec).  Everything that reads the layer's
+    normed input is ONE matrix in_w [sum of segments, width]; `seg` maps a segment name to its
+    (first column, width) in that projection's output:
+      delta layer:     q | k | v | b | a | g
+      parallel layer:  lq | lk | lv | lg (window attention and its per-head gate), then
+                       q | k | v | b | a1 | g1 of the delta mixer (a1 / g1: the low-rank inputs of
+                       decay and gate, widened by a2 / g2)
+    q | k | v of the delta mixer are adjacent so that one convolution launch covers them (conv_w
+    [q + k + v channels, taps]).  Per-head numbers and everything the recurrence reads besides the
+    projections are float32."""
+    norm1: torch.Tensor
+    norm2: Optional[torch.Tensor]
+    in_w: torch.Tensor
+    seg: dict
+    conv_w: torch.Tensor
+    a_log: torch.Tensor                     # f32 [heads]
+    dt_bias: torch.Tensor                   # f32 [heads] or [heads * dim]
+    head_norm: torch.Tensor                 # f32 [vdim]
+    delta_o_w: torch.Tensor
+    a2_w: Optional[torch.Tensor] = None     # [heads * dim, rank]
+    g2_w: Optional[torch.Tensor] = None     # [heads * vdim, rank]
+    attn_temp: Optional[torch.Tensor] = None    # f32 [heads]
+    attn_bias: Optional[torch.Tensor] = None    # f32 [heads]
+    attn_o_w: Optional[torch.Tensor] = None
+    attn_out_norm: Optional[torch.Tensor] = None
+    delta_out_norm: Optional[torch.Tensor] = None
+    gate_up_w: Optional[torch.Tensor] = None    # [2 ff, width]
+    down_w: Optional[torch.Tensor] = None       # [width, ff]
+
+    def tensors(self):
+        return [t for t in vars(self).values() if isinstance(t, torch.Tensor)]
+
+
+@dataclass
 class ModelWeights:
     embed: torch.Tensor
     layers: list = field(default_factory=list)
@@ -76,17 +111,18 @@ class ModelWeights:
     synthetic: bool = False
     pos_embed: Optional[torch.Tensor] = None     # learned positions (OPT): [max_positions + offset, hidden]
     final_norm_b: Optional[torch.Tensor] = None
+    loop_step: Optional[torch.Tensor] = None     # hybrid decoders with a loop: [passes, width]
 
     def nbytes(self) -> int:
         total = self.embed.numel() * self.embed.element_size()
         if self.lm_head.untyped_storage().data_ptr() != self.embed.untyped_storage().data_ptr():
             total += self.lm_head.numel() * self.lm_head.element_size()
         total += self.final_norm.numel() * self.final_norm.element_size()
-        for t in (self.pos_embed, self.final_norm_b):
+        for t in (self.pos_embed, self.final_norm_b, self.loop_step):
             if t is not None:
                 total += t.numel() * t.element_size()
         for lw in self.layers:
-            ts = lw.tensors() if isinstance(lw, OPTLayerWeights) else \
+            ts = lw.tensors() if isinstance(lw, (OPTLayerWeights, HybridLayerWeights)) else \
                 (lw.qkv_w, lw.qkv_b, lw.o_w, lw.gate_up_w, lw.down_w, lw.input_norm, lw.post_norm)
             for t in ts:
                 if t is not None:
@@ -124,6 +160,8 @@ def from_getter(cfg: ModelConfig, get: Callable[[str], torch.Tensor], dtype: tor
     """``get(name)`` returns the full (unsharded) CPU tensor of an HF parameter."""
     if cfg.family == "opt":
         return _opt_from_getter(cfg, get, dtype, device, tp_size, num_layers)
+    if cfg.family == "hybrid":
+        return _hybrid_from_getter(cfg, get, dtype, device, tp_size, num_layers)
     _, _, qs, ks = _shard_heads(cfg, tp_rank, tp_size)
     fs = _shard_mlp(cfg, tp_rank, tp_size) if shard_mlp else slice(None)
 
@@ -224,6 +262,144 @@ def _opt_synthetic(cfg: ModelConfig, dtype, device, seed: int, tp_size: int, num
     return w
 
 
+def _hybrid_one_gpu(tp_size: int, num_layers) -> None:
+    if tp_size != 1:
+        raise ValueError("hybrid decoders run on one GPU (tensor_parallel_size 1)")
+    if num_layers is not None:
+        raise ValueError("hybrid decoders run all their layers (no layer override)")
+
+
+def _hybrid_from_getter(cfg: ModelConfig, get, dtype, device, tp_size: int, num_layers) -> ModelWeights:
+    """Lozupel checkpoints: 'embed', 'head', 'final.norm', 'loop.step', and per layer i 'l<i>.norm1',
+    'l<i>.norm2', 'l<i>.mix.*' (a parallel layer's two mixers under '.left' / '.right'),
+    'l<i>.mlp.gate|up|down'.  Linear weights are [out, in]."""
+    _hybrid_one_gpu(tp_size, num_layers)
+    spec = cfg.hybrid
+    W = cfg.hidden_size
+
+    def put(t, dt=dtype):
+        return t.to(dt).contiguous().to(device)
+
+    def f32(t):
+        return put(t.reshape(-1), torch.float32)
+
+    def fuse(parts):
+        seg, at = {}, 0
+        for name, t in parts:
+            if t.dim() != 2 or t.shape[1] != W:
+                raise ValueError(f"segment {name}: shape {tuple(t.shape)}, expected [*, {W}]")
+            seg[name] = (at, int(t.shape[0]))
+            at += -(-int(t.shape[0]) // 8) * 8          # every segment starts on a 16-byte boundary of the output row
+        full = torch.zeros(at, W, dtype=parts[0][1].dtype)
+        for name, t in parts:
+            full[seg[name][0]: seg[name][0] + seg[name][1]] = t
+        return put(full), seg
+
+    def expect(name, t, shape):
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t
+
+    w = ModelWeights(embed=put(expect("embed", get("embed"), (cfg.vocab_size, W))))
+    for i, L in enumerate(spec.layers):
+        p = f"l{i}."
+        m = p + "mix." + ("right." if L.kind == "parallel" else "")
+        D = L.delta
+        qk, vv = D.kv_heads * D.dim, D.heads * D.vdim
+        parts = []
+        if L.kind == "parallel":
+            A, a = L.attn, p + "mix.left."
+            parts += [("lq", expect(a + "q", get(a + "q"), (A.heads * A.dim, W))),
+                      ("lk", expect(a + "k", get(a + "k"), (A.kv_heads * A.dim, W))),
+                      ("lv", expect(a + "v", get(a + "v"), (A.kv_heads * A.vdim, W))),
+                      ("lg", expect(a + "g", get(a + "g"), (A.heads, W)))]
+        parts += [("q", expect(m + "q", get(m + "q"), (qk, W))), ("k", expect(m + "k", get(m + "k"), (qk, W))),
+                  ("v", expect(m + "v", get(m + "v"), (vv, W))), ("b", expect(m + "b", get(m + "b"), (D.heads, W)))]
+        if D.per_channel:
+            parts += [("a1", get(m + "a1")), ("g1", get(m + "g1"))]
+        else:
+            parts += [("a", expect(m + "a", get(m + "a"), (D.heads, W))), ("g", expect(m + "g", get(m + "g"), (vv, W)))]
+        in_w, seg = fuse(parts)
+        conv = torch.cat([expect(m + n + ".conv", get(m + n + ".conv"), (c, D.conv))
+                          for n, c in (("q", qk), ("k", qk), ("v", vv))], dim=0)
+        lw = HybridLayerWeights(
+            norm1=put(get(p + "norm1").reshape(1)), norm2=put(get(p + "norm2").reshape(1)) if L.ff else None,
+            in_w=in_w, seg=seg, conv_w=put(conv), a_log=f32(expect(m + "A_log", get(m + "A_log"), (D.heads,))),
+            dt_bias=f32(expect(m + "dt_bias", get(m + "dt_bias"), (D.heads * D.dim if D.per_channel else D.heads,))),
+            head_norm=f32(expect(m + "norm", get(m + "norm"), (D.vdim,))),
+            delta_o_w=put(expect(m + "o", get(m + "o"), (W, vv))))
+        if D.per_channel:
+            lw.a2_w = put(expect(m + "a2", get(m + "a2"), (D.heads * D.dim, seg["a1"][1])))
+            lw.g2_w = put(expect(m + "g2", get(m + "g2"), (vv, seg["g1"][1])))
+        if L.kind == "parallel":
+            A, a = L.attn, p + "mix.left."
+            lw.attn_temp, lw.attn_bias = f32(expect(a + "temp", get(a + "temp"), (A.heads,))), \
+                f32(expect(a + "pb", get(a + "pb"), (A.heads,)))
+            lw.attn_o_w = put(expect(a + "o", get(a + "o"), (W, A.heads * A.vdim)))
+            lw.attn_out_norm = put(expect(a + "out", get(a + "out"), (W,)))
+            lw.delta_out_norm = put(expect(m + "out", get(m + "out"), (W,)))
+        if L.ff:
+            g, u = get(p + "mlp.gate"), get(p + "mlp.up")
+            lw.gate_up_w = put(torch.cat([expect(p + "mlp.gate", g, (L.ff, W)), expect(p + "mlp.up", u, (L.ff, W))], dim=0))
+            lw.down_w = put(expect(p + "mlp.down", get(p + "mlp.down"), (W, L.ff)))
+        w.layers.append(lw)
+    w.final_norm = put(get("final.norm").reshape(1))
+    w.lm_head = put(expect("head", get("head"), (cfg.vocab_size, W)))
+    if spec.loop_times > 0:
+        w.loop_step = put(expect("loop.step", get("loop.step"), (spec.loop_times, W)))
+    return w
+
+
+def hybrid_synthetic_state(cfg: ModelConfig, seed: int = 0, std: float = 0.02, rank: int = 32, device="cpu",
+                           dtype=torch.float32) -> dict:
+    """Seeded random tensors under a Lozupel checkpoint's names (benchmarks and tests: nothing can be
+    downloaded).  `rank`: the inner width of the low-rank decay / gate projections."""
+    spec, W = cfg.hybrid, cfg.hidden_size
+    gen = torch.Generator(device=device).manual_seed(seed)
+
+    def mat(*shape, s=std):
+        return torch.empty(shape, dtype=dtype, device=device).normal_(0.0, s, generator=gen)
+
+    def near(value, *shape, s=0.1):
+        return torch.full(shape, float(value), dtype=dtype, device=device) + mat(*shape, s=s)
+
+    st = {"embed": mat(cfg.vocab_size, W, s=1.0), "head": mat(cfg.vocab_size, W), "final.norm": near(1.0)}
+    if spec.loop_times > 0:
+        st["loop.step"] = mat(spec.loop_times, W, s=0.1)
+    for i, L in enumerate(spec.layers):
+        p = f"l{i}."
+        st[p + "norm1"] = near(1.0)
+        m = p + "mix." + ("right." if L.kind == "parallel" else "")
+        D = L.delta
+        qk, vv = D.kv_heads * D.dim, D.heads * D.vdim
+        for n, c in (("q", qk), ("k", qk), ("v", vv)):
+            st[m + n] = mat(c, W, s=W ** -0.5)
+            st[m + n + ".conv"] = mat(c, D.conv, s=D.conv ** -0.5)
+        st[m + "b"] = mat(D.heads, W, s=W ** -0.5)
+        st[m + "A_log"] = mat(D.heads, s=0.5)
+        st[m + "norm"] = near(1.0, D.vdim)
+        st[m + "o"] = mat(W, vv, s=vv ** -0.5)
+        if D.per_channel:
+            st[m + "a1"], st[m + "a2"] = mat(rank, W, s=W ** -0.5), mat(D.heads * D.dim, rank, s=rank ** -0.5)
+            st[m + "g1"], st[m + "g2"] = mat(rank, W, s=W ** -0.5), mat(vv, rank, s=rank ** -0.5)
+            st[m + "dt_bias"] = mat(D.heads * D.dim, s=0.5)
+        else:
+            st[m + "a"], st[m + "g"] = mat(D.heads, W, s=W ** -0.5), mat(vv, W, s=W ** -0.5)
+            st[m + "dt_bias"] = mat(D.heads, s=0.5)
+        if L.kind == "parallel":
+            A, a = L.attn, p + "mix.left."
+            st[a + "q"], st[a + "k"] = mat(A.heads * A.dim, W, s=W ** -0.5), mat(A.kv_heads * A.dim, W, s=W ** -0.5)
+            st[a + "v"], st[a + "g"] = mat(A.kv_heads * A.vdim, W, s=W ** -0.5), mat(A.heads, W, s=W ** -0.5)
+            st[a + "temp"], st[a + "pb"] = near(1.0, A.heads), near(-2.0, A.heads, s=0.5)
+            st[a + "o"] = mat(W, A.heads * A.vdim, s=(A.heads * A.vdim) ** -0.5)
+            st[a + "out"], st[m + "out"] = near(1.0, W), near(1.0, W)
+        if L.ff:
+            st[p + "norm2"] = near(1.0)
+            st[p + "mlp.gate"], st[p + "mlp.up"] = mat(L.ff, W, s=W ** -0.5), mat(L.ff, W, s=W ** -0.5)
+            st[p + "mlp.down"] = mat(W, L.ff, s=L.ff ** -0.5)
+    return st
+
+
 def from_state_dict(cfg, state: dict, dtype, device, **kw) -> ModelWeights:
     def get(name):
         t = state[name]
@@ -270,6 +446,12 @@ def synthetic(cfg: ModelConfig, dtype, device, seed: int = 0, tp_rank: int = 0, 
     replicated tensors from the same stream so they are bit-identical across ranks."""
     if cfg.family == "opt":
         return _opt_synthetic(cfg, dtype, device, seed, tp_size, num_layers, std)
+    if cfg.family == "hybrid":
+        _hybrid_one_gpu(tp_size, num_layers)
+        state = hybrid_synthetic_state(cfg, seed=seed, device=device)
+        w = from_state_dict(cfg, state, dtype, device)
+        w.synthetic = True
+        return w
     nh_l, nkv_l, _, _ = _shard_heads(cfg, tp_rank, tp_size)
     H, F, V, d = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.head_dim
     if shard_mlp:
