@@ -210,3 +210,69 @@ def forward(w, cfg, tokens, trace=None):
     if cap:
         z = cap * torch.tanh(z / cap)
     return z
+
+
+def random_state(cfg, seed=0, rank=5, bf16_grid=True):
+    """Seeded random tensors under the checkpoint names of `cfg` (a config dict), float32; with
+    bf16_grid every value is representable in bfloat16, so a 16-bit and a 32-bit run see the same
+    weights.  Scales keep activations O(1) through the layers."""
+    g = torch.Generator().manual_seed(seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def mat(*shape, s=1.0, mean=0.0):
+        t = torch.randn(tuple(shape), generator=g) * s + mean
+        return t.to(torch.bfloat16).float() if bf16_grid else t
+
+    st = {"embed": mat(V, W), "head": mat(V, W, s=W ** -0.5), "final.norm": mat(s=0.1, mean=1.0)}
+    if cfg.get("loop"):
+        st["loop.step"] = mat(cfg["loop"]["times"], W, s=0.3)
+
+    def delta(p, m, per_channel):
+        qk, vv = m["kv_heads"] * m["dim"], m["heads"] * m["vdim"]
+        for n, c in (("q", qk), ("k", qk), ("v", vv)):
+            st[p + n] = mat(c, W, s=W ** -0.5)
+            st[p + n + ".conv"] = mat(c, m["conv"], s=0.7)
+        st[p + "b"] = mat(m["heads"], W, s=W ** -0.5)
+        st[p + "A_log"] = mat(m["heads"], s=0.5, mean=-1.0)
+        st[p + "norm"] = mat(m["vdim"], s=0.2, mean=1.0)
+        st[p + "o"] = mat(W, vv, s=vv ** -0.5)
+        if per_channel:
+            st[p + "a1"], st[p + "a2"] = mat(rank, W, s=W ** -0.5), mat(m["heads"] * m["dim"], rank, s=1.0)
+            st[p + "g1"], st[p + "g2"] = mat(rank, W, s=W ** -0.5), mat(vv, rank, s=1.0)
+            st[p + "dt_bias"] = mat(m["heads"] * m["dim"], s=0.5)
+        else:
+            st[p + "a"], st[p + "g"] = mat(m["heads"], W, s=W ** -0.5), mat(vv, W, s=W ** -0.5)
+            st[p + "dt_bias"] = mat(m["heads"], s=0.5)
+
+    for i, L in enumerate(cfg["layers"]):
+        p = f"l{i}."
+        st[p + "norm1"] = mat(s=0.1, mean=1.0)
+        if L["type"] == "delta":
+            delta(p + "mix.", L["mixer"], False)
+        else:
+            a, m = p + "mix.left.", L["mixer"]["left"]
+            st[a + "q"] = mat(m["heads"] * m["dim"], W, s=W ** -0.5)
+            st[a + "k"] = mat(m["kv_heads"] * m["dim"], W, s=W ** -0.5)
+            st[a + "v"] = mat(m["kv_heads"] * m["vdim"], W, s=W ** -0.5)
+            st[a + "g"] = mat(m["heads"], W, s=W ** -0.5)
+            st[a + "temp"], st[a + "pb"] = mat(m["heads"], s=0.3, mean=1.0), mat(m["heads"], s=0.5, mean=-1.0)
+            st[a + "o"] = mat(W, m["heads"] * m["vdim"], s=(m["heads"] * m["vdim"]) ** -0.5)
+            st[a + "out"] = mat(W, s=0.2, mean=1.0)
+            delta(p + "mix.right.", L["mixer"]["right"], True)
+            st[p + "mix.right.out"] = mat(W, s=0.2, mean=1.0)
+        if L.get("mlp") is not None:
+            F_ = L["mlp"]["ff"]
+            st[p + "norm2"] = mat(s=0.1, mean=1.0)
+            st[p + "mlp.gate"], st[p + "mlp.up"] = mat(F_, W, s=W ** -0.5), mat(F_, W, s=W ** -0.5)
+            st[p + "mlp.down"] = mat(W, F_, s=F_ ** -0.5)
+    return st
+
+
+def greedy(w, cfg, prompt, steps):
+    """Greedy continuation of one prompt by full recomputation; returns (tokens, their logits rows)."""
+    toks, rows = list(prompt), []
+    for _ in range(steps):
+        z = forward(w, cfg, toks)[-1]
+        rows.append(z)
+        toks.append(int(torch.argmax(z)))
+    return toks[len(prompt):], torch.stack(rows)

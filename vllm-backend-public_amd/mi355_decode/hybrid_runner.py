@@ -156,7 +156,15 @@ class HybridRunner(ModelRunner):
         B = self.max_num_seqs
         self._init_step_inputs(extra_i32=1)
         self.row_extra.fill_(self.num_state_slots)
-        self.logits = torch.zeros(B, self.V, dtype=dtype, device=dev)
+        # the samplers want 16-byte aligned logit rows: the head is padded with zero rows to a multiple
+        # of 8 and the logits are the first V columns of what it yields
+        self.Vp = -(-self.V // 8) * 8
+        self.head_w = weights.lm_head
+        if self.Vp != self.V:
+            self.head_w = torch.zeros(self.Vp, self.H, dtype=dtype, device=dev)
+            self.head_w[: self.V] = weights.lm_head
+        self.logits_rows = torch.zeros(B, self.Vp, dtype=dtype, device=dev)
+        self.logits = self.logits_rows[:, : self.V]
         self.graphs = {}
         self.buckets = batch_buckets(B)
         self._init_step_staging()
@@ -247,21 +255,18 @@ class HybridRunner(ModelRunner):
     def _logits(self, resid: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Final norm, head and soft cap over the given residual rows."""
         h = ops.add_rms_norm_f32(resid, self.w.final_norm, self.eps)
-        z = self.linear(h, self.w.lm_head, out=out)
+        z = self.linear(h, self.head_w, out=out)
         if self.spec.logit_softcap:
             ops.softcap(z, self.spec.logit_softcap)
-        return z
+        return z[:, : self.V]
 
     # ------------------------------------------------------------------ #
     def _decode_body(self, b: int) -> None:
         batch = StepBatch(self.ids[:b], self.positions[:b], self.slots[:b], self.block_tables[:b],
                           self._dec_cu[:b + 1], self._dec_seq[:b], self.row_extra[:b])
         resid = self._forward(batch)
-        self._logits(resid, out=self.logits[:b])
+        self._logits(resid, out=self.logits_rows[:b])
         self.greedy(self.logits[:b], self.next_ids[:b], ids_out=self.ids[:b])
-
-    def lm_head_logits(self, x: torch.Tensor, out: torch.Tensor) -> None:
-        self.linear(x, self.w.lm_head, out=out)
 
     def run_prefill(self, token_ids, positions, slot_mapping, block_tables, cu_seqlens, context_lens, max_q_len: int,
                     sampling: Optional[dict] = None, logprobs: int = -1, prompt_logprobs=None, state_slots=None,

@@ -969,6 +969,8 @@ def resid_add_f32(resid: torch.Tensor, other: torch.Tensor | None = None, rows: 
     """resid (float32, in place) += other (float32 rows) + rows (activation rows) + vec (one row)."""
     T, W = resid.shape
     dt = None
+    if T == 0:
+        return resid
     for name, t, shape in (("rows", rows, (T, W)), ("vec", vec, (W,))):
         if t is None:
             continue
@@ -1075,7 +1077,9 @@ def rope_partial_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos
         raise ValueError("K pages must be [blocks, kv_heads, 16, head_dim] and V pages [blocks, kv_heads, 16, v_dim]")
     check(lib.mi355_rope_partial_kv_write(
         q.data_ptr(), _cols(q, "q", num_heads * head_dim), _same(k, q, "k"), _cols(k, "k", num_kv_heads * head_dim),
-        _same(v, q, "v"), _cols(v, "v", num_kv_heads * v_dim), _f32(cos_sin, "cos_sin"), cos_sin.shape[0],
+        _same(v, q, "v"), _cols(v, "v", num_kv_heads * v_dim),
+        _f32(cos_sin, "cos_sin") or q.data_ptr(),            # rot_dims 0: the table is empty and never read
+        max(cos_sin.shape[0], 1),
         _idx(positions, "positions", torch.int64, T), _idx(slot_mapping, "slot_mapping", torch.int64, T),
         _same(k_cache, q, "k_cache"), _same(v_cache, q, "v_cache"), T, num_heads, num_kv_heads, head_dim, v_dim, rot,
         dt, _stream()))
@@ -1120,10 +1124,11 @@ def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor,
     if out is None:
         out = torch.empty(T, C, dtype=x.dtype, device=x.device)
     args = (_idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(state_slots, "state_slots", torch.int32, S))
+    st = _f32(state, "state") or x.data_ptr()                # one tap: the state is empty and never read
     check(lib.mi355_causal_conv_silu(out.data_ptr(), x.data_ptr(), _cols(x, "x", C), weight.data_ptr(),
-                                     _f32(state, "state"), _idx(tok_seq, "tok_seq", torch.int32, T),
+                                     st, _idx(tok_seq, "tok_seq", torch.int32, T),
                                      _idx(positions, "positions", torch.int64, T), *args, T, C, taps, dt, _stream()))
-    check(lib.mi355_conv_state_update(state.data_ptr(), x.data_ptr(), _cols(x, "x", C), *args, S, C, taps, dt,
+    check(lib.mi355_conv_state_update(st, x.data_ptr(), _cols(x, "x", C), *args, S, C, taps, dt,
                                       _stream()))
     return out
 
