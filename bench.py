@@ -138,6 +138,12 @@ def parse():
                     help="timed regions of exactly --steps steps each; the median one is reported")
     ap.add_argument("--no-served", action="store_true", help="skip the measurement through the HTTP server")
     ap.add_argument("--served-runs", type=int, default=5)
+    ap.add_argument("--hybrid-compare", action="store_true",
+                    help="instead of the default workload: prefill and decode throughput of hybrid (Lozupel) decoders at a "
+                         "few real layer sizes beside Llama-shaped decoders of equal size, and the hybrid kernels' times "
+                         "against their rooflines beside the like kernels of the Llama path (random weights)")
+    ap.add_argument("--hybrid-widths", default="2048,4096")
+    ap.add_argument("--hybrid-layers", type=int, default=4)
     return ap.parse_args()
 
 
@@ -599,6 +605,11 @@ def pmc_traffic(tiled):
 
 def main():
     a = parse()
+    if a.hybrid_compare:
+        from mi355_decode.bench_hybrid import compare
+        print(json.dumps(compare([int(w) for w in a.hybrid_widths.split(",")], a.hybrid_layers, a.batch_per_gpu,
+                                 a.prompt_len if a.prompt_len != 128 else 2048, min(a.steps, 64), a.warmup)), flush=True)
+        return
     if a.gpus > 1 and "WORLD_SIZE" not in os.environ:
         # no launcher above us: become the parent of a.gpus rank processes (nothing GPU-related has
         # been imported yet) and relay rank 0's line

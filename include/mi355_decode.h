@@ -771,7 +771,7 @@ int32_t mi355_softcap(void* z, int64_t numel, float cap, int32_t dtype, void* st
  * Sequence mixers over a packed batch of chunks (whole prompts, portions of prompts and single
  * decoded tokens side by side): tok_seq[t] names the chunk of packed row t, positions[t] its
  * position in its sequence, cu_seqlens[s] the first row of chunk s.  K pages are
- * [blocks, kv_heads, 16, head_dim], V pages [blocks, kv_heads, 16, v_dim]; convolution state is
+ * [blocks, kv_heads, 16, head_dim], V pages [blocks, kv_heads, v_dim, 16]; convolution state is
  * fp32 [slots, taps - 1, channels], delta-rule state fp32 [slots, heads, head_dim, v_dim].
  *   rope_partial_kv_write  rotates the first rot_dims coordinates of every q and k head (coordinate
  *                          i with i + rot_dims / 2) by the fp32 table cos_sin [max_pos, rot_dims]
@@ -779,7 +779,13 @@ int32_t mi355_softcap(void* z, int64_t numel, float cap, int32_t dtype, void* st
  *                          rows with slot < 0 store nothing
  *   sigmoid_window_attn    out[t, h] = sigmoid(gate[t, h]) * sum over keys j of the row's sequence with
  *                          0 <= p - j < window of sigmoid(q.k_j * scale * temp[h] + bias[h]) * v_j
- *                          (gate may be null); weights are not normalised over keys
+ *                          (gate may be null); weights are not normalised over keys.  With `tiles`
+ *                          ([num_tiles][3] = chunk, first packed row, rows <= 16, covering every row
+ *                          once, positions consecutive inside a tile), 16-bit storage, head_dim a
+ *                          multiple of 32 and v_dim of 16, the products run on the matrix cores; there,
+ *                          with `partial` (fp32 [num_splits][num_tokens * num_heads * v_dim]) and
+ *                          num_splits > 1, the keys of a tile are dealt out to num_splits workgroups
+ *                          whose sums a second launch adds (few rows, long windows: decode)
  *   causal_conv_silu       y[t, c] = silu(sum_j w[c, j] * x[t - (taps - 1 - j), c]); inputs from before
  *                          the chunk come from the sequence's state slot, zeros before position 0
  *   conv_state_update      state slot <- the last taps - 1 inputs of each sequence (after the conv)
@@ -788,8 +794,13 @@ int32_t mi355_softcap(void* z, int64_t numel, float cap, int32_t dtype, void* st
  *                          unit vectors (q also / sqrt(head_dim)), b = sigmoid(beta),
  *                          a = exp(-exp(a_log[h]) * softplus(decay + dt_bias)), one per head
  *                          (per_channel 0) or one per key channel (per_channel 1: decay rows
- *                          [heads * head_dim]); q / k / v are columns q_off / k_off / v_off of qkv rows
+ *                          [heads * head_dim]); q / k / v are columns q_off / k_off / v_off of qkv rows.
+ *                          With a workspace of mi355_gated_delta_rule_workspace(...) floats the form for
+ *                          chunks of many tokens runs (state rows split over 8 lanes, per-token vectors
+ *                          prepared for all tokens first); without, one state column per lane (decode)
  */
+int64_t mi355_gated_delta_rule_workspace(int64_t num_tokens, int32_t num_heads, int32_t num_kv_heads,
+                                         int32_t head_dim);
 int32_t mi355_rope_partial_kv_write(void* q, int64_t q_stride, const void* k, int64_t k_stride,
                                     const void* v, int64_t v_stride, const float* cos_sin,
                                     int32_t max_pos, const int64_t* positions,
@@ -803,7 +814,8 @@ int32_t mi355_sigmoid_window_attn(void* out, const void* q, int64_t q_stride, co
                                   const int64_t* positions, const float* temp, const float* bias,
                                   const void* gate, int64_t gate_stride, int64_t num_tokens,
                                   int32_t num_heads, int32_t num_kv_heads, int32_t head_dim,
-                                  int32_t v_dim, int32_t window, float scale, int32_t dtype,
+                                  int32_t v_dim, int32_t window, float scale, const int32_t* tiles,
+                                  int32_t num_tiles, float* partial, int32_t num_splits, int32_t dtype,
                                   void* stream);
 int32_t mi355_causal_conv_silu(void* y, const void* x, int64_t x_stride, const void* weight,
                                const float* state, const int32_t* tok_seq, const int64_t* positions,
@@ -820,8 +832,9 @@ int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t stride, int32_
                                const float* dt_bias, int32_t per_channel, float* state,
                                const int32_t* cu_seqlens, const int64_t* positions,
                                const int32_t* state_slots, int32_t num_seqs, int32_t num_heads,
-                               int32_t num_kv_heads, int32_t head_dim, int32_t v_dim, int32_t dtype,
-                               void* stream);
+                               int32_t num_kv_heads, int32_t head_dim, int32_t v_dim,
+                               int64_t num_tokens, float* workspace, int64_t workspace_floats,
+                               int32_t dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -154,7 +154,7 @@ def _paged(T, num_pages, seed):
     return order, order[pos // 16].astype(np.int64) * 16 + pos % 16
 
 
-def _attend_in_cuts(q, k, v, cuts, H, G, d, dv, window, rot, temp, bias, gate, scale=0.3, base=100.0):
+def _attend_in_cuts(q, k, v, cuts, H, G, d, dv, window, rot, temp, bias, gate, scale=0.3, base=100.0, tiled=False):
     """rope + store + attention over one sequence fed in portions; returns [T, H * dv] float32."""
     from mi355_decode import ops
     from mi355_decode.hybrid_runner import rotary_table
@@ -163,7 +163,7 @@ def _attend_in_cuts(q, k, v, cuts, H, G, d, dv, window, rot, temp, bias, gate, s
     pages = 12
     table, slots = _paged(T, pages, 5)
     kc = torch.full((pages, G, 16, d), float("nan"), dtype=dt, device="cuda")
-    vc = torch.full((pages, G, 16, dv), float("nan"), dtype=dt, device="cuda")
+    vc = torch.full((pages, G, dv, 16), float("nan"), dtype=dt, device="cuda")
     bt = torch.zeros(1, pages, dtype=torch.int32)
     bt[0, : len(table)] = torch.from_numpy(table)
     cs = rotary_table(rot, base, pages * 16, "cuda")
@@ -176,7 +176,11 @@ def _attend_in_cuts(q, k, v, cuts, H, G, d, dv, window, rot, temp, bias, gate, s
                                   H, G, d, dv)
         outs.append(ops.sigmoid_window_attn(qq, kc, vc, bt.cuda(), torch.zeros(n, dtype=torch.int32, device="cuda"), pos,
                                             temp.cuda(), bias.cuda(), None if gate is None else gate[sl].cuda(), H,
-                                            window, scale).float().cpu())
+                                            window, scale,
+                                            tiles=torch.from_numpy(ops.query_tiles([0, n])).cuda() if tiled else None,
+                                            # single rows: the window's keys spread over three workgroups
+                                            partial=torch.empty(3 * H * dv, device="cuda") if tiled and n == 1 else None,
+                                            num_splits=3 if tiled and n == 1 else 1).float().cpu())
         at += n
     assert at == T
     return torch.cat(outs)
@@ -199,6 +203,28 @@ def test_window_attention_whole_portions_and_single_tokens(H, G, d, dv, window, 
         assert (got - ref).abs().max() <= 2e-5 * ref.abs().max(), cuts
 
 
+@pytest.mark.parametrize("H,G,d,dv,window,rot", [(4, 2, 32, 48, 20, 16), (2, 1, 128, 64, 33, 128), (8, 2, 64, 64, 200, 32),
+                                                 (16, 1, 96, 16, 7, 64)])
+def test_window_attention_on_the_matrix_cores(H, G, d, dv, window, rot):
+    """The 16-row tile form (16-bit storage) against the restatement run on the same rounded inputs:
+    whole prompt, uneven portions, single rows; unused page slots hold NaN and must not leak."""
+    g = torch.Generator().manual_seed(H + d)
+    T = 75
+    bf = lambda t: t.to(torch.bfloat16)                                      # noqa: E731
+    q, k, v = bf(torch.randn(T, H * d, generator=g)), bf(torch.randn(T, G * d, generator=g)), bf(torch.randn(T, G * dv, generator=g))
+    temp, bias, gate = torch.rand(H, generator=g) + 0.5, torch.randn(H, generator=g) - 1.0, bf(torch.randn(T, H, generator=g))
+    pos = torch.arange(T)
+    qr = bf(R.rotate_partial(q.float().view(T, H, d), pos, rot, 100.0)).float()
+    kr = bf(R.rotate_partial(k.float().view(T, G, d), pos, rot, 100.0)).float()
+    ref = R.sigmoid_window_attention(qr, kr, v.float().view(T, G, dv), window, 0.3, temp, bias) \
+        * torch.sigmoid(gate.float())[:, :, None]
+    ref = ref.reshape(T, H * dv)
+    for cuts in ([T], [5, 16, 1, 17, 33, 3], [1] * 20 + [55]):
+        got = _attend_in_cuts(q, k, v, cuts, H, G, d, dv, window, rot, temp, bias, gate, tiled=True)
+        assert torch.isfinite(got).all()
+        assert (got - ref).abs().max() <= 1.5e-2 * ref.abs().max(), cuts
+
+
 @pytest.mark.parametrize("window", [16, 17, 31, 48])
 def test_window_edge_shows_with_one_loud_key(window):
     """One key far louder than the rest: the token window - 1 after it still hears it, the next one
@@ -213,13 +239,15 @@ def test_window_edge_shows_with_one_loud_key(window):
     v = torch.zeros(T, dv)
     v[j0, 3] = 1.0
     temp, bias = torch.ones(1), torch.full((1,), -30.0)          # every other key weighs sigmoid(-30)
-    for cuts in ([T], [j0 + 2] + [1] * (T - j0 - 2)):
-        got = _attend_in_cuts(q, k, v, cuts, H, G, d, dv, window, 0, temp, bias, None, scale=1.0)
+    for cuts, dt in (([T], torch.float32), ([j0 + 2] + [1] * (T - j0 - 2), torch.float32), ([T], torch.bfloat16),
+                     ([3, 40, T - 43], torch.bfloat16)):
+        got = _attend_in_cuts(q.to(dt), k.to(dt), v.to(dt), cuts, H, G, d, dv, window, 0, temp, bias, None, scale=1.0,
+                              tiled=dt == torch.bfloat16)
         inside, outside = j0 + window - 1, j0 + window
         assert got[inside, 3] > 0.99 and abs(got[outside, 3]) < 1e-6 and got[j0, 3] > 0.99 and got[j0 - 1, 3] == 0
 
 
-def _delta_in_cuts(qkv, beta, decay, a_log, dt_bias, cuts, H, G, d, dv, per_channel, slot=2, slots=4):
+def _delta_in_cuts(qkv, beta, decay, a_log, dt_bias, cuts, H, G, d, dv, per_channel, slot=2, slots=4, long_chunks=False):
     from mi355_decode import ops
     T = qkv.shape[0]
     state = torch.full((slots, H, d, dv), float("nan"), device="cuda")
@@ -232,7 +260,7 @@ def _delta_in_cuts(qkv, beta, decay, a_log, dt_bias, cuts, H, G, d, dv, per_chan
                                          torch.tensor([0, n], dtype=torch.int32, device="cuda"),
                                          torch.arange(at, at + n, dtype=torch.int64, device="cuda"),
                                          torch.tensor([slot], dtype=torch.int32, device="cuda"), H, G, d, dv,
-                                         per_channel=per_channel).cpu())
+                                         per_channel=per_channel, long_chunks=long_chunks and n > 1).cpu())
         at += n
     return torch.cat(outs)
 
@@ -259,8 +287,9 @@ def test_delta_rule_whole_portions_and_single_tokens(H, G, d, dv, per_channel):
     a_log, dt_bias = torch.randn(H, generator=g) * 0.5 - 1, torch.randn(decay.shape[1], generator=g) * 0.5
     ref = _delta_ref(qkv, beta, decay, a_log, dt_bias, H, G, d, dv, per_channel)
     for cuts in ([T], [1] * T, [2, 3, 1, 17, 2, 16]):
-        got = _delta_in_cuts(qkv, beta, decay, a_log, dt_bias, cuts, H, G, d, dv, per_channel)
-        assert (got - ref).abs().max() <= 3e-5 * ref.abs().max(), cuts
+        for long_chunks in (False, True):             # one column per lane; rows split over lanes (single tokens: always the former)
+            got = _delta_in_cuts(qkv, beta, decay, a_log, dt_bias, cuts, H, G, d, dv, per_channel, long_chunks=long_chunks)
+            assert (got - ref).abs().max() <= 3e-5 * ref.abs().max(), (cuts, long_chunks)
 
 
 def test_delta_rule_keeps_a_far_write_and_loses_it_with_decay():
@@ -277,7 +306,8 @@ def test_delta_rule_keeps_a_far_write_and_loses_it_with_decay():
     beta = torch.full((T, 1), 30.0)          # sigmoid -> 1
     for z, want in ((-40.0, 1.0), (1.0, 0.0)):
         decay = torch.full((T, 1), z)
-        got = _delta_in_cuts(qkv, beta, decay, torch.zeros(1), torch.zeros(1), [250] + [1] * 50, H, G, d, dv, False)
+        got = _delta_in_cuts(qkv, beta, decay, torch.zeros(1), torch.zeros(1), [250] + [1] * 50, H, G, d, dv, False,
+                             long_chunks=True)
         ref = _delta_ref(qkv, beta, decay, torch.zeros(1), torch.zeros(1), H, G, d, dv, False)
         assert (got - ref).abs().max() <= 1e-5
         assert abs(float(got[-1, 0, 7]) * d ** 0.5 - want) < 1e-3

@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void rope_partial_kv_write_kernel(
   }
   for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
     const int g = i / dv, j = i % dv;
-    MI355_ST(typename Elem<T>::S, v_cache, v_cache + ((page * G + g) * kPage + off) * dv + j,
+    MI355_ST(typename Elem<T>::S, v_cache, v_cache + ((page * G + g) * dv + j) * kPage + off,
              MI355_LD(typename Elem<T>::S, v, v + t * v_stride + static_cast<int64_t>(g) * dv + j));
   }
 }
@@ -112,12 +112,12 @@ __global__ __launch_bounds__(64) void sigmoid_window_attn_kernel(
     for (int jj = 0; jj < n; ++jj) {
       const int64_t key = base + jj;
       const int64_t page = MI355_LD(int32_t, block_tables, bt + key / kPage);
-      const typename Elem<T>::S* vr = v_cache + ((page * G + g) * kPage + key % kPage) * dv;
+      const typename Elem<T>::S* vr = v_cache + (page * G + g) * dv * kPage + key % kPage;
       const float wj = ws[jj];
 #pragma unroll
       for (int i = 0; i < DV_PER_LANE; ++i) {
         const int c = lane + 64 * i;
-        if (c < dv) acc[i] += wj * MI355_LDF(T, v_cache, vr + c);
+        if (c < dv) acc[i] += wj * MI355_LDF(T, v_cache, vr + c * kPage);
       }
     }
     __syncthreads();
@@ -128,6 +128,121 @@ __global__ __launch_bounds__(64) void sigmoid_window_attn_kernel(
   for (int i = 0; i < DV_PER_LANE; ++i) {
     const int c = lane + 64 * i;
     if (c < dv) MI355_STF(T, out, out + (t * H + h) * dv + c, acc[i] * gt);
+  }
+}
+
+// The matrix-core form for 16-bit activations, d a multiple of 32, dv a multiple of 16.  One
+// workgroup per (tile of up to 16 consecutive rows of one chunk, kv head); its waves take the
+// query heads of the group, so the K / V fragments they all read stay in the CU's cache.  Keys are
+// taken 32 at a time (two pages).  Scores are computed transposed, S^T = K Q^T, so that a lane ends
+// up holding, for its query (lane % 16), eight weights -- keys 4 (lane / 16) + r of either page --
+// which is exactly an A-operand fragment of the P V product once V's fragment lists the same
+// eight keys: with V pages stored [dv, 16 tokens] that is two 8-byte loads.  Scores, the sigmoid
+// and the accumulators are fp32; the weights are rounded to the storage type for the second product.
+template <typename T>
+__global__ __launch_bounds__(512) void sigmoid_window_attn_mfma_kernel(
+    uint16_t* __restrict__ out, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ k_cache,
+    const uint16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ tiles, const int64_t* __restrict__ positions, const float* __restrict__ temp,
+    const float* __restrict__ bias, const uint16_t* __restrict__ gate, int64_t gate_stride, int H, int G, int d, int dv,
+    int window, float scale, float* __restrict__ partial, int64_t partial_stride) {
+  constexpr int kMaxD = 256 / 32, kMaxDV = 256 / 16;
+  // gridDim.z > 1: the key tiles are dealt out to the z blocks in turn and each writes its fp32 sums
+  // (no gate) to its slab of `partial`; the weights are not normalised, so the slabs simply add up
+  const int nz = gridDim.z, z = blockIdx.z;
+  const int tile = blockIdx.x, g = blockIdx.y, rep = H / G;
+  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6, lane = threadIdx.x & 63;
+  const int li = lane & 15, kk = lane >> 4;
+  const int seq = MI355_LD(int32_t, tiles, tiles + 3 * tile);
+  const int64_t row0 = MI355_LD(int32_t, tiles, tiles + 3 * tile + 1);
+  const int nrows = MI355_LD(int32_t, tiles, tiles + 3 * tile + 2);
+  const int64_t p0 = MI355_LD(int64_t, positions, positions + row0);
+  const int32_t* bt = block_tables + static_cast<int64_t>(seq) * max_blocks;
+  const int ds = d >> 5, cbs = dv >> 4;
+  const int64_t p_last = p0 + nrows - 1;
+  int64_t lo = p0 - window + 1;
+  if (lo < 0) lo = 0;
+  const int64_t my_p = p0 + li;                       // position of this lane's query (rows past nrows: masked out)
+  for (int hh = wave; hh < rep; hh += nwaves) {
+    const int h = g * rep + hh;
+    uint4 qf[kMaxD];
+#pragma unroll
+    for (int s = 0; s < kMaxD; ++s) {
+      qf[s] = make_uint4(0, 0, 0, 0);
+      if (s < ds && li < nrows)
+        qf[s] = MI355_LD(uint4, q, q + (row0 + li) * q_stride + static_cast<int64_t>(h) * d + 32 * s + 8 * kk);
+    }
+    const float mul = scale * MI355_LD(float, temp, temp + h), add = MI355_LD(float, bias, bias + h);
+    f32x4 acc[kMaxDV];
+#pragma unroll
+    for (int c = 0; c < kMaxDV; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int64_t base = ((lo >> 5) << 5) + 32 * z; base <= p_last; base += 32 * nz) {
+      uint32_t pw[4];                                   // 8 weights of this lane's query, packed
+      int64_t pages[2];
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int64_t kb = base + 16 * half;
+        f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
+        pages[half] = -1;
+        if (kb <= p_last) {
+          pages[half] = MI355_LD(int32_t, block_tables, bt + kb / kPage);
+          const uint16_t* kr = k_cache + ((pages[half] * G + g) * kPage + li) * d + 8 * kk;
+#pragma unroll
+          for (int s = 0; s < kMaxD; ++s)
+            if (s < ds) sacc = T::mfma(MI355_LD(uint4, k_cache, kr + 32 * s), qf[s], sacc);
+        }
+        float w[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int64_t key = kb + 4 * kk + r;
+          const bool vis = li < nrows && key <= my_p && my_p - key < window;
+          w[r] = vis ? __frcp_rn(1.0f + __expf(-(sacc[r] * mul + add))) : 0.f;
+        }
+        pw[2 * half] = T::pack2(w[0], w[1]);
+        pw[2 * half + 1] = T::pack2(w[2], w[3]);
+      }
+      const uint4 pf = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+#pragma unroll
+      for (int c = 0; c < kMaxDV; ++c) {
+        if (c < cbs) {
+          uint2 v0 = make_uint2(0, 0), v1 = make_uint2(0, 0);
+          if (pages[0] >= 0)
+            v0 = MI355_LD(uint2, v_cache, v_cache + ((pages[0] * G + g) * dv + 16 * c + li) * kPage + 4 * kk);
+          if (pages[1] >= 0)
+            v1 = MI355_LD(uint2, v_cache, v_cache + ((pages[1] * G + g) * dv + 16 * c + li) * kPage + 4 * kk);
+          // slots past the newest key may hold anything (0 * NaN is NaN): clear them in the last tile
+          if (base + 31 > p_last) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+              uint2& vv = half == 0 ? v0 : v1;
+              const int64_t k0 = base + 16 * half + 4 * kk;
+              if (k0 > p_last) vv.x &= 0xFFFF0000u;
+              if (k0 + 1 > p_last) vv.x &= 0x0000FFFFu;
+              if (k0 + 2 > p_last) vv.y &= 0xFFFF0000u;
+              if (k0 + 3 > p_last) vv.y &= 0x0000FFFFu;
+            }
+          }
+          acc[c] = T::mfma(pf, make_uint4(v0.x, v0.y, v1.x, v1.y), acc[c]);
+        }
+      }
+    }
+    // C layout: this lane holds rows 4 kk + r of column li of every 16-column block
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int rr = 4 * kk + r;
+      if (rr >= nrows) continue;
+      if (partial != nullptr) {
+#pragma unroll
+        for (int c = 0; c < kMaxDV; ++c)
+          if (c < cbs) MI355_ST(float, partial, partial + z * partial_stride + ((row0 + rr) * H + h) * dv + 16 * c + li, acc[c][r]);
+        continue;
+      }
+      float gt = 1.0f;
+      if (gate != nullptr) gt = 1.0f / (1.0f + expf(-T::to_f(MI355_LD(uint16_t, gate, gate + (row0 + rr) * gate_stride + h))));
+#pragma unroll
+      for (int c = 0; c < kMaxDV; ++c)
+        if (c < cbs) MI355_ST(uint16_t, out, out + ((row0 + rr) * H + h) * dv + 16 * c + li, T::from_f(acc[c][r] * gt));
+    }
   }
 }
 
@@ -272,6 +387,170 @@ __global__ __launch_bounds__(64) void gated_delta_rule_kernel(
   }
 }
 
+// ---- the gated delta rule for chunks of many tokens -------------------------------------------------
+// With one state column per lane a token costs 4 * d dependent vector operations per wave and a
+// prompt keeps only heads * dv / 64 waves busy.  Here the d rows of a column are split over R = 8
+// adjacent lanes (a wave holds 8 columns, DR = ceil(d / 8) rows each), the two dot products of a
+// token are finished with three cross-lane steps each, and everything that does not depend on the
+// state -- unit-length key and query, decay, beta -- is computed for all tokens at once by
+// delta_prep_kernel, in fp32, into rows padded to 8 * DR (key / query 0, decay 1 in the padding).
+// The loop then reads the next token's rows while it works on the current one.
+constexpr int kSplit = 8;
+
+template <typename T>
+__global__ __launch_bounds__(64) void delta_prep_kernel(
+    float* __restrict__ kq, float* __restrict__ dec, float* __restrict__ bet, const typename Elem<T>::S* __restrict__ qkv,
+    int64_t stride, int q_off, int k_off, const typename Elem<T>::S* __restrict__ beta, int64_t beta_stride,
+    const typename Elem<T>::S* __restrict__ decay, int64_t decay_stride, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, int per_channel, int H, int G, int d, int dp) {
+  const int64_t t = blockIdx.x;
+  const int y = blockIdx.y, lane = threadIdx.x;
+  if (y < G) {                                          // unit-length key and scaled unit-length query of kv head y
+    const typename Elem<T>::S* row = qkv + t * stride;
+    float kk = 0.f, qq = 0.f;
+    for (int c = lane; c < d; c += 64) {
+      const float kv = MI355_LDF(T, qkv, row + k_off + y * d + c), qv = MI355_LDF(T, qkv, row + q_off + y * d + c);
+      kk += kv * kv;
+      qq += qv * qv;
+    }
+    kk = 1.0f / sqrtf(wave_sum(kk) + 1e-6f);
+    qq = (1.0f / sqrtf(static_cast<float>(d))) / sqrtf(wave_sum(qq) + 1e-6f);
+    float* o = kq + (t * G + y) * 2 * dp;
+    for (int c = lane; c < dp; c += 64) {
+      MI355_ST(float, kq, o + c, c < d ? MI355_LDF(T, qkv, row + k_off + y * d + c) * kk : 0.f);
+      MI355_ST(float, kq, o + dp + c, c < d ? MI355_LDF(T, qkv, row + q_off + y * d + c) * qq : 0.f);
+    }
+    return;
+  }
+  const int h = y - G;
+  const float na = -expf(MI355_LD(float, a_log, a_log + h));
+  float* o = dec + (t * H + h) * dp;
+  for (int c = lane; c < dp; c += 64) {
+    float a = 1.0f;
+    if (c < d) {
+      const float z = per_channel
+                          ? MI355_LDF(T, decay, decay + t * decay_stride + h * d + c) + MI355_LD(float, dt_bias, dt_bias + h * d + c)
+                          : MI355_LDF(T, decay, decay + t * decay_stride + h) + MI355_LD(float, dt_bias, dt_bias + h);
+      a = expf(na * (z > 20.0f ? z : log1pf(expf(z))));
+    }
+    MI355_ST(float, dec, o + c, a);
+  }
+  if (lane == 0)
+    MI355_ST(float, bet, bet + t * H + h, 1.0f / (1.0f + expf(-MI355_LDF(T, beta, beta + t * beta_stride + h))));
+}
+
+template <typename T, int DR, int PF>
+__global__ __launch_bounds__(64) void gated_delta_rule_split_kernel(
+    float* __restrict__ o, const typename Elem<T>::S* __restrict__ qkv, int64_t stride, int v_off,
+    const float* __restrict__ kq, const float* __restrict__ dec, const float* __restrict__ bet, float* __restrict__ state,
+    const int32_t* __restrict__ cu_seqlens, const int64_t* __restrict__ positions,
+    const int32_t* __restrict__ state_slots, int H, int G, int d, int dv) {
+  constexpr int dp = kSplit * DR;
+  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int r = lane & (kSplit - 1), col = blockIdx.z * (64 / kSplit) + (lane >> 3);
+  const int g = h / (H / G);
+  const int64_t cs = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s);
+  const int64_t n = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1) - cs;
+  if (n <= 0) return;
+  const int64_t slot = MI355_LD(int32_t, state_slots, state_slots + s);
+  float* sp = state + ((slot * H + h) * d) * dv;
+  const bool live = col < dv;
+  const bool fresh = MI355_LD(int64_t, positions, positions + cs) == 0;
+  float S[DR];
+#pragma unroll
+  for (int j = 0; j < DR; ++j) {
+    const int i = r * DR + j;
+    S[j] = (live && !fresh && i < d) ? MI355_LD(float, state, sp + static_cast<int64_t>(i) * dv + col) : 0.f;
+  }
+  // the rows of the next PF tokens travel while the current PF tokens are worked on: a token's
+  // arithmetic is far shorter than a trip to memory
+  float nk[PF][DR], nq[PF][DR], na[PF][DR], nb[PF], nv[PF];
+  auto fetch = [&](int64_t first) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      int64_t t = first + u;
+      if (t > cs + n - 1) t = cs + n - 1;               // past the chunk: a row that is loaded and not used
+      const float* kp = kq + (t * G + g) * 2 * dp + r * DR;
+      const float* ap = dec + (t * H + h) * dp + r * DR;
+#pragma unroll
+      for (int j = 0; j < DR; j += 4) {
+        const float4 a4 = MI355_LD(float4, kq, kp + j), b4 = MI355_LD(float4, kq, kp + dp + j), c4 = MI355_LD(float4, dec, ap + j);
+        nk[u][j] = a4.x, nk[u][j + 1] = a4.y, nk[u][j + 2] = a4.z, nk[u][j + 3] = a4.w;
+        nq[u][j] = b4.x, nq[u][j + 1] = b4.y, nq[u][j + 2] = b4.z, nq[u][j + 3] = b4.w;
+        na[u][j] = c4.x, na[u][j + 1] = c4.y, na[u][j + 2] = c4.z, na[u][j + 3] = c4.w;
+      }
+      nb[u] = MI355_LD(float, bet, bet + t * H + h);
+      nv[u] = live ? MI355_LDF(T, qkv, qkv + t * stride + v_off + h * dv + col) : 0.f;
+    }
+  };
+  fetch(cs);
+  for (int64_t i0 = 0; i0 < n; i0 += PF) {
+    float k[PF][DR], q[PF][DR], a[PF][DR], b[PF], vj[PF];
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+#pragma unroll
+      for (int j = 0; j < DR; ++j) k[u][j] = nk[u][j], q[u][j] = nq[u][j], a[u][j] = na[u][j];
+      b[u] = nb[u], vj[u] = nv[u];
+    }
+    if (i0 + PF < n) fetch(cs + i0 + PF);
+#pragma unroll
+    for (int u = 0; u < PF; ++u) {
+      if (i0 + u >= n) break;
+      float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+      for (int j = 0; j < DR; j += 2) {
+        S[j] *= a[u][j];
+        S[j + 1] *= a[u][j + 1];
+        d0 += S[j] * k[u][j];
+        d1 += S[j + 1] * k[u][j + 1];
+      }
+      float dot = d0 + d1;
+      dot += __shfl_xor(dot, 1, 64);
+      dot += __shfl_xor(dot, 2, 64);
+      dot += __shfl_xor(dot, 4, 64);
+      const float uu = b[u] * (vj[u] - dot);
+      float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int j = 0; j < DR; j += 2) {
+        S[j] += k[u][j] * uu;
+        S[j + 1] += k[u][j + 1] * uu;
+        o0 += S[j] * q[u][j];
+        o1 += S[j + 1] * q[u][j + 1];
+      }
+      float out = o0 + o1;
+      out += __shfl_xor(out, 1, 64);
+      out += __shfl_xor(out, 2, 64);
+      out += __shfl_xor(out, 4, 64);
+      if (live && r == 0) MI355_ST(float, o, o + ((cs + i0 + u) * H + h) * dv + col, out);
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < DR; ++j) {
+      const int i = r * DR + j;
+      if (i < d) MI355_ST(float, state, sp + static_cast<int64_t>(i) * dv + col, S[j]);
+    }
+  }
+}
+
+// out = sigmoid(gate) * sum of the key-range partial sums of sigmoid_window_attn_mfma_kernel
+template <typename T>
+__global__ __launch_bounds__(256) void window_attn_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial,
+                                                                 const uint16_t* __restrict__ gate, int64_t gate_stride,
+                                                                 int64_t rows, int H, int dv, int splits) {
+  const int64_t total = rows * H * dv;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    float v = 0.f;
+    for (int z = 0; z < splits; ++z) v += MI355_LD(float, partial, partial + z * total + i);
+    const int64_t th = i / dv;
+    float gt = 1.0f;
+    if (gate != nullptr)
+      gt = 1.0f / (1.0f + expf(-T::to_f(MI355_LD(uint16_t, gate, gate + (th / H) * gate_stride + th % H))));
+    MI355_ST(uint16_t, out, out + i, T::from_f(v * gt));
+  }
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -333,7 +612,8 @@ extern "C" int32_t mi355_sigmoid_window_attn(void* out, const void* q, int64_t q
                                              const float* bias, const void* gate, int64_t gate_stride,
                                              int64_t num_tokens, int32_t num_heads, int32_t num_kv_heads,
                                              int32_t head_dim, int32_t v_dim, int32_t window, float scale,
-                                             int32_t dtype, void* stream) {
+                                             const int32_t* tiles, int32_t num_tiles, float* partial,
+                                             int32_t num_splits, int32_t dtype, void* stream) {
   MI355_REQUIRE(out && q && k_cache && v_cache && block_tables && tok_seq && positions && temp && bias,
                 MI355_ERR_INVALID, "sigmoid_window_attn: null pointer");
   MI355_REQUIRE(num_tokens >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0 &&
@@ -344,6 +624,29 @@ extern "C" int32_t mi355_sigmoid_window_attn(void* out, const void* q, int64_t q
   REQ_DTYPE(dtype);
   if (num_tokens == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (tiles != nullptr && num_tiles > 0 && dtype != MI355_F32 && head_dim % 32 == 0 && head_dim <= 256 &&
+      v_dim % 16 == 0 && q_stride % 8 == 0 && aligned16(q) && aligned16(k_cache) && aligned16(v_cache)) {
+    // the matrix-core form: `tiles` lists (chunk, first row, rows <= 16) for every 16-row tile of the batch
+    const int rep = num_heads / num_kv_heads;
+    const bool split = partial != nullptr && num_splits > 1;
+    MI355_REQUIRE(num_splits >= 0 && num_splits <= 64, MI355_ERR_INVALID, "sigmoid_window_attn: %d key splits", num_splits);
+    const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(num_kv_heads), split ? num_splits : 1);
+    const dim3 block(64u * static_cast<unsigned>(rep < 8 ? rep : 8));
+    const int64_t slab = num_tokens * num_heads * v_dim;
+#define MI355_WMFMA(TT)                                                                                             \
+  hipLaunchKernelGGL((sigmoid_window_attn_mfma_kernel<TT>), grid, block, 0, s, static_cast<uint16_t*>(out),          \
+                     static_cast<const uint16_t*>(q), q_stride, static_cast<const uint16_t*>(k_cache),               \
+                     static_cast<const uint16_t*>(v_cache), block_tables, max_blocks, tiles, positions, temp, bias,  \
+                     static_cast<const uint16_t*>(gate), gate_stride, num_heads, num_kv_heads, head_dim, v_dim,      \
+                     window, scale, split ? partial : nullptr, slab);                                                \
+  if (split)                                                                                                        \
+    hipLaunchKernelGGL((window_attn_reduce_kernel<TT>), dim3(static_cast<unsigned>((slab + 255) / 256 > 4096 ? 4096 : (slab + 255) / 256)), \
+                       dim3(256), 0, s, static_cast<uint16_t*>(out), partial, static_cast<const uint16_t*>(gate),    \
+                       gate_stride, num_tokens, num_heads, v_dim, num_splits)
+    if (dtype == MI355_BF16) { MI355_WMFMA(BF16); } else { MI355_WMFMA(F16); }
+#undef MI355_WMFMA
+    return check_launch("sigmoid_window_attn (matrix cores)");
+  }
   MI355_DISPATCH_DTYPE3(dtype, launch_window_attn<TT>(s, out, q, q_stride, k_cache, v_cache, block_tables, max_blocks,
                                                      tok_seq, positions, temp, bias, gate, gate_stride, num_tokens,
                                                      num_heads, num_kv_heads, head_dim, v_dim, window, scale));
@@ -404,12 +707,19 @@ static void launch_delta(hipStream_t s, float* o, const void* qkv, int64_t strid
 #undef MI355_DELTA
 }
 
+extern "C" int64_t mi355_gated_delta_rule_workspace(int64_t num_tokens, int32_t num_heads, int32_t num_kv_heads,
+                                                    int32_t head_dim) {
+  const int64_t dp = 8 * (head_dim <= 32 ? 4 : head_dim <= 64 ? 8 : head_dim <= 128 ? 16 : 32);
+  return num_tokens * (static_cast<int64_t>(num_kv_heads) * 2 * dp + static_cast<int64_t>(num_heads) * dp + num_heads + 4) / 4 * 4;
+}
+
 extern "C" int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t stride, int32_t q_off, int32_t k_off,
                                           int32_t v_off, const void* beta, int64_t beta_stride, const void* decay,
                                           int64_t decay_stride, const float* a_log, const float* dt_bias,
                                           int32_t per_channel, float* state, const int32_t* cu_seqlens,
                                           const int64_t* positions, const int32_t* state_slots, int32_t num_seqs,
                                           int32_t num_heads, int32_t num_kv_heads, int32_t head_dim, int32_t v_dim,
+                                          int64_t num_tokens, float* workspace, int64_t workspace_floats,
                                           int32_t dtype, void* stream) {
   MI355_REQUIRE(o && qkv && beta && decay && a_log && dt_bias && state && cu_seqlens && positions && state_slots,
                 MI355_ERR_INVALID, "gated_delta_rule: null pointer");
@@ -421,6 +731,34 @@ extern "C" int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t str
   REQ_DTYPE(dtype);
   if (num_seqs == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (workspace != nullptr && num_tokens > 0) {
+    // the form for chunks of many tokens: rows split over 8 lanes, per-token vectors prepared up front
+    const int dr = head_dim <= 32 ? 4 : head_dim <= 64 ? 8 : head_dim <= 128 ? 16 : 32;
+    const int64_t dp = 8 * dr;
+    const int64_t need = mi355_gated_delta_rule_workspace(num_tokens, num_heads, num_kv_heads, head_dim);
+    MI355_REQUIRE(workspace_floats >= need && aligned16(workspace), MI355_ERR_INVALID,
+                  "gated_delta_rule: workspace of %lld floats, %lld needed, 16-byte aligned",
+                  static_cast<long long>(workspace_floats), static_cast<long long>(need));
+    float* kq = workspace;
+    float* dec = kq + num_tokens * num_kv_heads * 2 * dp;
+    float* bet = dec + num_tokens * num_heads * dp;
+    const dim3 pgrid(static_cast<unsigned>(num_tokens), static_cast<unsigned>(num_kv_heads + num_heads));
+    const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>((v_dim + 7) / 8));
+#define MI355_DSPLIT(TT, DR)                                                                                          \
+  hipLaunchKernelGGL((gated_delta_rule_split_kernel<TT, DR, (DR <= 16 ? 4 : 2)>), grid, dim3(64), 0, s, o,            \
+                     static_cast<const Elem<TT>::S*>(qkv), stride, v_off, kq, dec, bet, state, cu_seqlens, positions, \
+                     state_slots, num_heads, num_kv_heads, head_dim, v_dim)
+    MI355_DISPATCH_DTYPE3(dtype, {
+      hipLaunchKernelGGL((delta_prep_kernel<TT>), pgrid, dim3(64), 0, s, kq, dec, bet, static_cast<const Elem<TT>::S*>(qkv),
+                         stride, q_off, k_off, static_cast<const Elem<TT>::S*>(beta), beta_stride,
+                         static_cast<const Elem<TT>::S*>(decay), decay_stride, a_log, dt_bias, per_channel, num_heads,
+                         num_kv_heads, head_dim, static_cast<int>(dp));
+      if (dr == 4) MI355_DSPLIT(TT, 4); else if (dr == 8) MI355_DSPLIT(TT, 8); else if (dr == 16) MI355_DSPLIT(TT, 16);
+      else MI355_DSPLIT(TT, 32);
+    });
+#undef MI355_DSPLIT
+    return check_launch("gated_delta_rule (split rows)");
+  }
   MI355_DISPATCH_DTYPE3(dtype, launch_delta<TT>(s, o, qkv, stride, q_off, k_off, v_off, beta, beta_stride, decay,
                                                decay_stride, a_log, dt_bias, per_channel, state, cu_seqlens, positions,
                                                state_slots, num_seqs, num_heads, num_kv_heads, head_dim, v_dim));

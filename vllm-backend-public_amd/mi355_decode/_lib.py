@@ -106,11 +106,12 @@ def _load() -> ctypes.CDLL:
         "mi355_rope_partial_kv_write": (I32, [P, I64, P, I64, P, I64, P, I32, P, P, P, P, I64, I32, I32, I32, I32, I32,
                                               I32, P]),
         "mi355_sigmoid_window_attn": (I32, [P, P, I64, P, P, P, I32, P, P, P, P, P, I64, I64, I32, I32, I32, I32, I32,
-                                            F, I32, P]),
+                                            F, P, I32, P, I32, I32, P]),
         "mi355_causal_conv_silu": (I32, [P, P, I64, P, P, P, P, P, P, I64, I32, I32, I32, P]),
         "mi355_conv_state_update": (I32, [P, P, I64, P, P, I32, I32, I32, I32, P]),
         "mi355_gated_delta_rule": (I32, [P, P, I64, I32, I32, I32, P, I64, P, I64, P, P, I32, P, P, P, P, I32, I32, I32,
-                                         I32, I32, I32, P]),
+                                         I32, I32, I64, P, I64, I32, P]),
+        "mi355_gated_delta_rule_workspace": (I64, [I64, I32, I32, I32]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
@@ -144,7 +145,7 @@ EXPORTS = ("mi355_abi_version", "mi355_last_error", "mi355_target_arch",
            "mi355_embed_scale_f32", "mi355_resid_add_f32", "mi355_add_rms_norm_f32", "mi355_rms_norm_mix_f32",
            "mi355_gelu_tanh_and_mul", "mi355_gated_head_rms_norm", "mi355_softcap",
            "mi355_rope_partial_kv_write", "mi355_sigmoid_window_attn", "mi355_causal_conv_silu",
-           "mi355_conv_state_update", "mi355_gated_delta_rule")
+           "mi355_conv_state_update", "mi355_gated_delta_rule", "mi355_gated_delta_rule_workspace")
 
 
 def check(status: int) -> None:

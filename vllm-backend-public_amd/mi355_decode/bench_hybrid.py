@@ -1,0 +1,227 @@
+"""`bench.py --hybrid-compare`: hybrid (Lozupel) decoders at a few real layer sizes beside
+Llama-shaped decoders of equal width, depth and parameter count, random weights.
+
+Two parts.  (1) Through the engine: prompt tokens per second (a batch of prompts, chunked by the
+scheduler) and decoded tokens per second (decode steps replayed from HIP graphs).  (2) Kernel by
+kernel: the hybrid path's kernels timed alone at the prefill and the decode shape, each against
+its own roofline (HBM bytes at 8 TB/s, bf16 MFMA at 2.5 PFLOP/s, or fp32 vector FMA at 157 TFLOP/s,
+whichever bounds it), beside the like kernel of the Llama path at the same shape."""
+from __future__ import annotations
+
+import time
+
+import numpy as np
+import torch
+
+from . import ops
+from ._lib import BLOCK_SIZE
+from .config import EngineArgs, ModelConfig
+
+HBM, MFMA, VALU = 8.0e12, 2.5e15, 157.3e12
+
+
+def lozupel_config(width: int, layers: int, vocab: int = 32000) -> dict:
+    """Alternating parallel / delta layers with 128-wide heads, a 1024-token window, a feed-forward in
+    every layer; the middle of the stack loops twice."""
+    nh = width // 128
+    left = {"heads": nh, "kv_heads": max(nh // 4, 1), "dim": 128, "vdim": 128, "mask": {"size": 1024},
+            "rot": {"dims": 64, "base": 1.0e6}, "scale": 128 ** -0.5}
+    right = {"heads": max(nh // 2, 1), "kv_heads": max(nh // 4, 1), "dim": 128, "vdim": 128, "conv": 4}
+    delta = {"heads": nh, "kv_heads": max(nh // 2, 1), "dim": 128, "vdim": 128, "conv": 4}
+    ff = {"kind": "dense", "ff": 2 * width}
+    ls = [({"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": ff} if i % 2 == 0 else
+           {"type": "delta", "mixer": delta, "mlp": ff}) for i in range(layers)]
+    d = {"architecture": "Lozupel", "embedding": {"scale": 1.0}, "width": width, "vocab": vocab, "norm": {"eps": 1e-6},
+         "logit_softcap": 30.0, "layers": ls}
+    if layers >= 3:
+        d["loop"] = {"start": 1, "stop": layers - 1, "times": 2}
+    return d
+
+
+def _params(weights) -> int:
+    return sum(t.numel() for lw in weights.layers for t in (lw.tensors() if hasattr(lw, "tensors") else
+                                                            (lw.qkv_w, lw.o_w, lw.gate_up_w, lw.down_w)))
+
+
+def llama_config(width: int, layer_runs: int, layer_params: int, vocab: int = 32000) -> dict:
+    """A Llama-shaped decoder of the same width and depth whose layers hold `layer_params` weights each."""
+    nh, nkv, d = width // 128, max(width // 512, 1), 128
+    attn = (nh + 2 * nkv) * d * width + nh * d * width
+    inter = max(int((layer_params - attn) / (3 * width)) // 256 * 256, 256)
+    return dict(architectures=["LlamaForCausalLM"], vocab_size=vocab, hidden_size=width, intermediate_size=inter,
+                num_hidden_layers=layer_runs, num_attention_heads=nh, num_key_value_heads=nkv, rope_theta=1.0e6,
+                rms_norm_eps=1e-6, max_position_embeddings=8192, tie_word_embeddings=False, torch_dtype="bfloat16")
+
+
+def through_engine(cfg: ModelConfig, batch: int, prompt_len: int, steps: int, warmup: int) -> dict:
+    from .llm import build_engine
+    from .sampling_params import SamplingParams
+    eng = build_engine(EngineArgs(model="synthetic", dtype="bfloat16", max_num_seqs=batch,
+                                  max_model_len=prompt_len + steps + warmup + 16, max_num_batched_tokens=8192,
+                                  load_format="dummy", gpu_memory_utilization=0.9, seed=0), model_config=cfg)
+    rng = np.random.default_rng(0)
+    out = {"params_per_layer": _params(eng.runner.w) // max(len(eng.runner.w.layers), 1)}
+    best = float("inf")
+    pb = min(batch, 4)
+    for rep in range(3):                                  # prompts: time from submission to every first token
+        for i in range(pb):
+            eng.add_request(f"p{rep}-{i}", rng.integers(0, cfg.vocab_size, prompt_len).tolist(),
+                            SamplingParams(max_tokens=1, temperature=0.0, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while eng.has_unfinished():
+            eng.step()
+        torch.cuda.synchronize()
+        best = min(best, time.perf_counter() - t0)
+    out["prefill_tok_s"] = round(pb * prompt_len / best, 1)
+    for i in range(batch):
+        eng.add_request(f"d{i}", rng.integers(0, cfg.vocab_size, prompt_len).tolist(),
+                        SamplingParams(max_tokens=warmup + steps + 8, temperature=0.0, ignore_eos=True))
+    while eng.stats["decode_steps"] < warmup:
+        eng.step()
+    torch.cuda.synchronize()
+    first, t0 = eng.stats["decode_steps"], time.perf_counter()
+    while eng.stats["decode_steps"] < first + steps:
+        eng.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    out["decode_ms_per_step"] = round(dt * 1e3 / steps, 4)
+    out["decode_tok_s"] = round(batch * steps / dt, 1)
+    out["decode_graphs"] = bool(eng.runner.graphs)
+    for rid in list(eng.seqs):
+        eng.abort_request(rid)
+    while eng._pending:
+        eng._harvest_decode()
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
+def _time(fn, reps: int = 20) -> float:
+    """Seconds per call: best of three event-timed runs of `reps` back-to-back launches."""
+    fn()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(3):
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(reps):
+            fn()
+        e.record()
+        e.synchronize()
+        best = min(best, s.elapsed_time(e) * 1e-3 / reps)
+    return best
+
+
+def kernel_table(width: int, prompt_len: int, batch: int) -> list:
+    """[{kernel, shape, us, bound, frac_of_roofline, like, like_us, like_frac}]"""
+    dev, bf = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rnd = lambda *s, dt=bf: torch.randn(*s, device=dev, dtype=torch.float32, generator=g).to(dt)  # noqa: E731
+    H, G, d, dv, window = width // 128, max(width // 512, 1), 128, 128, 1024
+    F = 2 * width
+    rows = []
+
+    def row(kernel, shape, t, bound, work, like=None, like_t=None, like_work=None):
+        peak = {"hbm": HBM, "mfma": MFMA, "valu": VALU}[bound]
+        r = {"kernel": kernel, "shape": shape, "us": round(t * 1e6, 2), "bound": bound,
+             "frac_of_roofline": round(work / peak / t, 4)}
+        if like is not None:
+            r.update(like=like, like_us=round(like_t * 1e6, 2), like_frac=round(like_work / peak / like_t, 4))
+        rows.append(r)
+
+    for T, tag in ((prompt_len, "prefill"), (batch, "decode")):
+        shape = f"{tag} {T} rows x {width}"
+        resid, add16, w1, wv = rnd(T, width, dt=torch.float32), rnd(T, width), rnd(1), rnd(width)
+        x16, r16, out16 = rnd(T, width), rnd(T, width), torch.empty(T, width, device=dev, dtype=bf)
+        row("add_rms_norm_f32 (one-number weight)", shape, _time(lambda: ops.add_rms_norm_f32(resid, w1, 1e-6, add=add16, out=out16)),
+            "hbm", T * width * 12, "fused_add_rms_norm", _time(lambda: ops.fused_add_rms_norm(x16, r16, wv, 1e-6, out=out16)),
+            T * width * 8)
+        xa, xb = rnd(T, width), rnd(T, width)
+        row("rms_norm_mix_f32", shape, _time(lambda: ops.rms_norm_mix_f32(resid, xa, wv, xb, wv, 1e-6, 0.5)), "hbm",
+            T * width * 12)
+        gu, act = rnd(T, 2 * F), torch.empty(T, F, device=dev, dtype=bf)
+        row("gelu_tanh_and_mul", f"{tag} {T} rows x {F}", _time(lambda: ops.gelu_tanh_and_mul(gu, out=act)), "hbm", T * F * 6,
+            "silu_and_mul", _time(lambda: ops.silu_and_mul(gu, out=act)), T * F * 6)
+
+    # ---- attention: one prompt of prompt_len tokens; then `batch` sequences decoding at that context
+    P = prompt_len
+    pages = (P + BLOCK_SIZE) // BLOCK_SIZE + 1
+    nb = pages * batch
+    kc, vct = rnd(nb, G, BLOCK_SIZE, d), rnd(nb, G, dv, BLOCK_SIZE)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev).view(batch, pages)
+    temp, bias = torch.ones(H, device=dev), torch.full((H,), -2.0, device=dev)
+    q, gate = rnd(P, H * d), rnd(P, H)
+    pos = torch.arange(P, dtype=torch.int64, device=dev)
+    seq0 = torch.zeros(P, dtype=torch.int32, device=dev)
+    cu, ctx = torch.tensor([0, P], dtype=torch.int32, device=dev), torch.tensor([P], dtype=torch.int32, device=dev)
+    o = torch.empty(P, H * dv, device=dev, dtype=bf)
+    keys = sum(min(i + 1, window) for i in range(P))
+    tiles = torch.from_numpy(ops.query_tiles([0, P])).to(dev)
+    t_h = _time(lambda: ops.sigmoid_window_attn(q, kc, vct, bt[:1], seq0, pos, temp, bias, gate, H, window, d ** -0.5, out=o,
+                                                tiles=tiles), 5)
+    t_l = _time(lambda: ops.paged_attn_prefill(q, kc, vct, bt[:1], cu, ctx, P, H, G, d, d ** -0.5, out=o), 5)
+    row("sigmoid_window_attn", f"prefill {P} tokens, window {window}, {H}/{G} heads x {d}", t_h, "mfma", 2.0 * keys * H * (d + dv),
+        "paged_attn_prefill (causal softmax)", t_l, 2.0 * (P * (P + 1) // 2) * H * 2 * d)
+    qd, gd = rnd(batch, H * d), rnd(batch, H)
+    posd = torch.full((batch,), P - 1, dtype=torch.int64, device=dev)
+    seqd = torch.arange(batch, dtype=torch.int32, device=dev)
+    ctxd = torch.full((batch,), P, dtype=torch.int32, device=dev)
+    od = torch.empty(batch, H * dv, device=dev, dtype=bf)
+    ws = torch.empty(max(ops.decode_workspace_bytes(batch, H, d, 16), 16), dtype=torch.uint8, device=dev)
+    dtiles = torch.stack([seqd, seqd, torch.ones_like(seqd)], dim=1).contiguous()
+    part = torch.empty(8 * batch * H * dv, device=dev)
+    t_h = _time(lambda: ops.sigmoid_window_attn(qd, kc, vct, bt, seqd, posd, temp, bias, gd, H, window, d ** -0.5, out=od,
+                                                tiles=dtiles, partial=part, num_splits=8))
+    t_l = _time(lambda: ops.paged_attn_decode(qd, kc, vct, bt, ctxd, H, G, d, d ** -0.5, num_splits=4, workspace=ws, out=od))
+    row("sigmoid_window_attn", f"decode {batch} rows at context {P}, window {window}", t_h, "hbm",
+        batch * min(P, window) * G * (d + dv) * 2, "paged_attn_decode (whole context)", t_l, batch * P * G * 2 * d * 2)
+
+    # ---- the recurrence: heads of 128 x 128 state
+    Hd, Gd = width // 128, max(width // 256, 1)
+    C = 2 * Gd * d + Hd * dv
+    for T, S, tag in ((P, 1, "prefill"), (batch, batch, "decode")):
+        x = rnd(T, C)
+        conv_w = rnd(C, 4)
+        cst = torch.zeros(S + 1, 3, C, device=dev)
+        st = torch.zeros(S + 1, Hd, d, dv, device=dev)
+        per = T // S
+        cu_ = torch.arange(0, T + 1, per, dtype=torch.int32, device=dev)
+        pos_ = (torch.arange(T, device=dev) % per + (0 if S == 1 else P)).to(torch.int64)
+        seq_ = (torch.arange(T, device=dev) // per).to(torch.int32)
+        slots = torch.arange(S, dtype=torch.int32, device=dev)
+        y = torch.empty(T, C, device=dev, dtype=bf)
+        row("causal_conv_silu + state update", f"{tag} {T} rows x {C} channels, 4 taps",
+            _time(lambda: ops.causal_conv_silu(x, conv_w, cst, seq_, pos_, cu_, slots, out=y)), "hbm", T * C * 4)
+        beta, dec = rnd(T, Hd), rnd(T, Hd)
+        a_log, dtb = torch.zeros(Hd, device=dev), torch.zeros(Hd, device=dev)
+        oo = torch.empty(T, Hd, dv, device=dev)
+        t = _time(lambda: ops.gated_delta_rule(x, 0, Gd * d, 2 * Gd * d, beta, dec, a_log, dtb, st, cu_, pos_, slots, Hd, Gd, d,
+                                               dv, out=oo, long_chunks=S == 1), 5)
+        if S == 1:
+            row("gated_delta_rule", f"prefill {T} tokens, {Hd} heads x {d} x {dv}", t, "valu", 6.0 * T * Hd * d * dv)
+        else:
+            row("gated_delta_rule", f"decode {S} rows, {Hd} heads x {d} x {dv}", t, "hbm", S * Hd * d * dv * 8)
+        gt, hn = rnd(T, Hd * dv), torch.ones(dv, device=dev)
+        on = torch.empty(T, Hd * dv, device=dev, dtype=bf)
+        row("gated_head_rms_norm", f"{tag} {T} rows x {Hd} heads x {dv}", _time(lambda: ops.gated_head_rms_norm(oo, gt, hn, 1e-6, 0, out=on)),
+            "hbm", T * Hd * dv * 8)
+    return rows
+
+
+def compare(widths, layers: int, batch: int, prompt_len: int, steps: int, warmup: int) -> dict:
+    result = {"metric": "hybrid_vs_llama_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+              "config": {"layers": layers, "batch": batch, "prompt_len": prompt_len, "decode_steps": steps},
+              "models": [], "kernels": {}}
+    for width in widths:
+        hc = ModelConfig.from_dict(lozupel_config(width, layers))
+        h = through_engine(hc, batch, prompt_len, steps, warmup)
+        runs = len(hc.hybrid.runs())
+        # equal size: as many layer runs, as many weights read per run
+        lc = ModelConfig.from_dict(llama_config(width, runs, h["params_per_layer"]))
+        ll = through_engine(lc, batch, prompt_len, steps, warmup)
+        result["models"].append({"width": width, "layer_runs": runs, "hybrid": h, "llama": ll,
+                                 "prefill_ratio": round(h["prefill_tok_s"] / ll["prefill_tok_s"], 3),
+                                 "decode_ratio": round(h["decode_tok_s"] / ll["decode_tok_s"], 3)})
+        result["kernels"][str(width)] = kernel_table(width, prompt_len, batch)
+    return result

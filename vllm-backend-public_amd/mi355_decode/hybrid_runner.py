@@ -7,7 +7,7 @@ What differs from ModelRunner's decoders, and where it lives:
   * the residual stream is float32 (csrc/resid32.hip: norms with one learned number or a vector,
     residual adds, the gelu-tanh gate, the logit soft cap); activations and weights are bfloat16
     (or float32 throughout with dtype float32: every kernel here is built for both);
-  * K/V pages hold rotated keys [blocks, kv_heads, 16, dim] and values [blocks, kv_heads, 16, vdim],
+  * K/V pages hold rotated keys [blocks, kv_heads, 16, dim] and values [blocks, kv_heads, vdim, 16],
     one pair per layer RUN (a looped layer has one per pass), on the engine's block tables;
   * recurrent and convolution state lives in per-sequence slots (engine.SlotAllocator), again one
     set per layer run; a chunk that starts at position 0 resets its slot;
@@ -43,9 +43,12 @@ def rotary_table(rot_dims: int, base: float, max_pos: int, device) -> torch.Tens
 class StepBatch:
     """Device-side description of one packed step (see csrc/seqmix.hip)."""
     __slots__ = ("ids", "positions", "slot_mapping", "block_tables", "cu_seqlens", "tok_seq", "state_slots",
-                 "num_tokens", "num_seqs")
+                 "num_tokens", "num_seqs", "tiles", "long_chunks")
 
-    def __init__(self, ids, positions, slot_mapping, block_tables, cu_seqlens, tok_seq, state_slots):
+    def __init__(self, ids, positions, slot_mapping, block_tables, cu_seqlens, tok_seq, state_slots, tiles=None,
+                 long_chunks=False):
+        self.tiles = tiles                            # 16-row query tiles (ops.query_tiles) or None: one wave per row
+        self.long_chunks = long_chunks                # some chunk holds several tokens (prompts and portions)
         self.ids, self.positions, self.slot_mapping, self.block_tables = ids, positions, slot_mapping, block_tables
         self.cu_seqlens, self.tok_seq, self.state_slots = cu_seqlens, tok_seq, state_slots
         self.num_tokens, self.num_seqs = int(ids.numel()), int(cu_seqlens.numel()) - 1
@@ -67,7 +70,8 @@ class WindowAttention:
         ops.rope_partial_kv_write(q, k, v, r.rotary(s.rot_dims, s.rot_base), b.positions, b.slot_mapping, kc, vc,
                                   s.heads, s.kv_heads, s.dim, s.vdim)
         o = ops.sigmoid_window_attn(q, kc, vc, b.block_tables, b.tok_seq, b.positions, self.lw.attn_temp,
-                                    self.lw.attn_bias, g, s.heads, s.window, s.scale)
+                                    self.lw.attn_bias, g, s.heads, s.window, s.scale, tiles=b.tiles,
+                                    **r.key_splits(b, s))
         return r.linear(o, self.lw.attn_o_w)
 
 
@@ -95,7 +99,7 @@ class DeltaMixer:
             gate = proj[:, seg["g"][0]: seg["g"][0] + vv]
         o = ops.gated_delta_rule(y, 0, qk, 2 * qk, beta, decay, lw.a_log, lw.dt_bias, rec_state, b.cu_seqlens,
                                  b.positions, b.state_slots, s.heads, s.kv_heads, s.dim, s.vdim,
-                                 per_channel=s.per_channel)
+                                 per_channel=s.per_channel, long_chunks=b.long_chunks)
         on = ops.gated_head_rms_norm(o, gate, lw.head_norm, r.eps, ops.ACT_SIGMOID if s.per_channel else ops.ACT_SILU)
         return r.linear(on, lw.delta_o_w)
 
@@ -145,7 +149,7 @@ class HybridRunner(ModelRunner):
             if L.attn is not None:
                 A = L.attn
                 self.k_cache.append(torch.zeros(self.num_blocks, A.kv_heads, BLOCK_SIZE, A.dim, dtype=dtype, device=dev))
-                self.v_cache.append(torch.zeros(self.num_blocks, A.kv_heads, BLOCK_SIZE, A.vdim, dtype=dtype, device=dev))
+                self.v_cache.append(torch.zeros(self.num_blocks, A.kv_heads, A.vdim, BLOCK_SIZE, dtype=dtype, device=dev))
                 attn = WindowAttention(A, lw, self, len(self.k_cache) - 1)
             chans = 2 * D.kv_heads * D.dim + D.heads * D.vdim
             self.conv_state.append(torch.zeros(self.num_state_slots + 1, max(D.conv - 1, 0), chans, dtype=torch.float32,
@@ -171,6 +175,10 @@ class HybridRunner(ModelRunner):
         # a decode step is B chunks of one row each
         self._dec_cu = torch.arange(B + 1, dtype=torch.int32, device=dev)
         self._dec_seq = torch.arange(B, dtype=torch.int32, device=dev)
+        # a decoded token is a tile of one row; its window's keys are spread over up to 8 workgroups
+        self._dec_tiles = torch.stack([self._dec_seq, self._dec_seq, torch.ones_like(self._dec_seq)], dim=1).contiguous()
+        widest = max([L.attn.heads * L.attn.vdim for L in spec.layers if L.attn is not None] + [0])
+        self._attn_partial = torch.empty(max(self.MAX_KEY_SPLITS * B * widest, 4), dtype=torch.float32, device=dev)
         self.layer_trace = None                       # a list: _forward appends the residual after every layer run
 
     # ------------------------------------------------------------------ #
@@ -179,6 +187,16 @@ class HybridRunner(ModelRunner):
         if key not in self._rotary:
             self._rotary[key] = rotary_table(rot_dims, base, self.max_blocks * BLOCK_SIZE, self.device)
         return self._rotary[key]
+
+    MAX_KEY_SPLITS = 8
+
+    def key_splits(self, b: StepBatch, a) -> dict:
+        """Workgroups per tile for the window attention: more than one only for batches of few rows
+        (decoded tokens), where one workgroup per row and kv head would leave most of the chip idle."""
+        if b.tiles is None or b.long_chunks or b.num_tokens > self.max_num_seqs:
+            return {}
+        n = min(self.MAX_KEY_SPLITS, max(a.window // 64, 1))
+        return {"partial": self._attn_partial, "num_splits": n} if n > 1 else {}
 
     def kv_cache_bytes_per_block(self) -> int:
         return sum(t[0].numel() * t.element_size() for t in self.k_cache + self.v_cache)
@@ -263,7 +281,7 @@ class HybridRunner(ModelRunner):
     # ------------------------------------------------------------------ #
     def _decode_body(self, b: int) -> None:
         batch = StepBatch(self.ids[:b], self.positions[:b], self.slots[:b], self.block_tables[:b],
-                          self._dec_cu[:b + 1], self._dec_seq[:b], self.row_extra[:b])
+                          self._dec_cu[:b + 1], self._dec_seq[:b], self.row_extra[:b], self._dec_tiles[:b])
         resid = self._forward(batch)
         self._logits(resid, out=self.logits_rows[:b])
         self.greedy(self.logits[:b], self.next_ids[:b], ids_out=self.ids[:b])
@@ -277,6 +295,9 @@ class HybridRunner(ModelRunner):
         if state_slots is None:
             raise ValueError("hybrid decoders need the state slot of every chunk")
         self._step_state_slots = np.asarray(state_slots, dtype=np.int32)
+        # rows go to the matrix cores in tiles of up to 16 rows of one chunk
+        self._step_tiles = ops.query_tiles(cu_seqlens)
+        self._step_long = int(max_q_len) > 1
         if logit_rows is None:
             return super().run_prefill(token_ids, positions, slot_mapping, block_tables, cu_seqlens, context_lens,
                                        max_q_len, sampling=sampling, logprobs=logprobs, prompt_logprobs=prompt_logprobs)
@@ -297,8 +318,9 @@ class HybridRunner(ModelRunner):
         tok_seq = torch.repeat_interleave(torch.arange(S, dtype=torch.int32, device=self.device), lens,
                                           output_size=int(token_ids.numel()))
         slots = torch.from_numpy(self._step_state_slots).to(self.device, non_blocking=True)
+        tiles = torch.from_numpy(self._step_tiles).to(self.device, non_blocking=True)
         return self._forward(StepBatch(token_ids, positions, slot_mapping, block_tables.contiguous(), cu_seqlens,
-                                       tok_seq, slots))
+                                       tok_seq, slots, tiles, self._step_long))
 
     def prefill(self, token_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor,
                 block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,

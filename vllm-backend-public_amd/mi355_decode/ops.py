@@ -1072,9 +1072,9 @@ def rope_partial_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos
     dt = _dt3(q, "q")
     T = q.shape[0]
     rot = cos_sin.shape[1]
-    if tuple(k_cache.shape[1:]) != (num_kv_heads, BLOCK_SIZE, head_dim) or tuple(v_cache.shape[1:]) != (num_kv_heads, BLOCK_SIZE, v_dim) \
+    if tuple(k_cache.shape[1:]) != (num_kv_heads, BLOCK_SIZE, head_dim) or tuple(v_cache.shape[1:]) != (num_kv_heads, v_dim, BLOCK_SIZE) \
             or k_cache.shape[0] != v_cache.shape[0] or not k_cache.is_contiguous() or not v_cache.is_contiguous():
-        raise ValueError("K pages must be [blocks, kv_heads, 16, head_dim] and V pages [blocks, kv_heads, 16, v_dim]")
+        raise ValueError("K pages must be [blocks, kv_heads, 16, head_dim] and V pages [blocks, kv_heads, v_dim, 16]")
     check(lib.mi355_rope_partial_kv_write(
         q.data_ptr(), _cols(q, "q", num_heads * head_dim), _same(k, q, "k"), _cols(k, "k", num_kv_heads * head_dim),
         _same(v, q, "v"), _cols(v, "v", num_kv_heads * v_dim),
@@ -1088,12 +1088,18 @@ def rope_partial_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos
 def sigmoid_window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                         tok_seq: torch.Tensor, positions: torch.Tensor, temp: torch.Tensor, bias: torch.Tensor,
                         gate: torch.Tensor | None, num_heads: int, window: int, scale: float,
-                        out: torch.Tensor | None = None):
+                        out: torch.Tensor | None = None, tiles: torch.Tensor | None = None,
+                        partial: torch.Tensor | None = None, num_splits: int = 1):
     """Sliding-window attention with sigmoid weights over the paged K/V of each packed row's
-    sequence.  Returns [tokens, heads * v_dim]."""
+    sequence.  Returns [tokens, heads * v_dim].  `tiles` (int32 [n, 3], see query_tiles) selects the
+    matrix-core form where the shapes allow it; there `partial` (float32, >= num_splits * tokens *
+    heads * v_dim elements) with num_splits > 1 spreads each tile's keys over num_splits workgroups."""
     dt = _dt3(q, "q")
     T = q.shape[0]
-    G, d, dv = k_cache.shape[1], k_cache.shape[3], v_cache.shape[3]
+    G, d, dv = k_cache.shape[1], k_cache.shape[3], v_cache.shape[2]
+    if tiles is not None and (tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 3
+                              or not tiles.is_contiguous() or not tiles.is_cuda):
+        raise ValueError("tiles must be a contiguous int32 [n, 3] tensor on the GPU")
     if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
         raise ValueError("block_tables must be contiguous int32 [chunks, max_blocks]")
     if out is None:
@@ -1104,8 +1110,24 @@ def sigmoid_window_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.T
         _idx(tok_seq, "tok_seq", torch.int32, T), _idx(positions, "positions", torch.int64, T),
         _f32(temp, "temp", num_heads), _f32(bias, "bias", num_heads),
         None if gate is None else _same(gate, q, "gate"), 0 if gate is None else _cols(gate, "gate", num_heads),
-        T, num_heads, G, d, dv, int(window), float(scale), dt, _stream()))
+        T, num_heads, G, d, dv, int(window), float(scale), None if tiles is None else tiles.data_ptr(),
+        0 if tiles is None else tiles.shape[0],
+        None if partial is None or num_splits <= 1 else _f32(partial[: num_splits * T * num_heads * dv], "partial",
+                                                             num_splits * T * num_heads * dv),
+        int(num_splits), dt, _stream()))
     return out
+
+
+def query_tiles(cu_seqlens) -> "np.ndarray":
+    """(chunk, first packed row, rows <= 16) for every 16-row tile of a packed batch, from the host
+    copy of cu_seqlens: the work list of the matrix-core window attention."""
+    import numpy as np
+    cu = np.asarray(cu_seqlens, dtype=np.int64)
+    out = []
+    for s in range(len(cu) - 1):
+        for a in range(int(cu[s]), int(cu[s + 1]), 16):
+            out.append((s, a, min(16, int(cu[s + 1]) - a)))
+    return np.asarray(out, dtype=np.int32).reshape(-1, 3)
 
 
 def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, tok_seq: torch.Tensor,
@@ -1136,12 +1158,14 @@ def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, state: torch.Tensor,
 def gated_delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, beta: torch.Tensor, decay: torch.Tensor,
                      a_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
                      positions: torch.Tensor, state_slots: torch.Tensor, num_heads: int, num_kv_heads: int,
-                     head_dim: int, v_dim: int, per_channel: bool = False, out: torch.Tensor | None = None):
+                     head_dim: int, v_dim: int, per_channel: bool = False, out: torch.Tensor | None = None,
+                     long_chunks: bool = False):
     """The gated delta rule over packed chunks.  qkv [tokens, C] holds q (kv_heads x head_dim) at column
     q_off, k at k_off, v (heads x v_dim) at v_off; beta [tokens, heads] and decay [tokens, heads] or
     [tokens, heads * head_dim] are raw projection outputs (column slices are fine); a_log [heads] and
     dt_bias (decay's width) float32; state float32 [slots, heads, head_dim, v_dim].
-    Returns o float32 [tokens, heads, v_dim]."""
+    Returns o float32 [tokens, heads, v_dim].  long_chunks: the batch holds chunks of many tokens -- take
+    the form that splits the state rows over lanes (it allocates a float32 workspace; not for graphs)."""
     dt = _dt3(qkv, "qkv")
     T = qkv.shape[0]
     S = cu_seqlens.numel() - 1
@@ -1153,10 +1177,15 @@ def gated_delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, beta
         raise ValueError("qkv must be contiguous [tokens, >= the q / k / v columns]")
     if out is None:
         out = torch.empty(T, num_heads, v_dim, dtype=torch.float32, device=qkv.device)
+    ws = None
+    if long_chunks and T > 0:
+        ws = torch.empty(lib.mi355_gated_delta_rule_workspace(T, num_heads, num_kv_heads, head_dim), dtype=torch.float32,
+                         device=qkv.device)
     check(lib.mi355_gated_delta_rule(
         _f32(out, "out", T * num_heads * v_dim), qkv.data_ptr(), qkv.shape[1], q_off, k_off, v_off,
         _same(beta, qkv, "beta"), _cols(beta, "beta", num_heads), _same(decay, qkv, "decay"), _cols(decay, "decay", width),
         _f32(a_log, "a_log", num_heads), _f32(dt_bias, "dt_bias", width), int(per_channel), _f32(state, "state"),
         _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(positions, "positions", torch.int64, T),
-        _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, num_kv_heads, head_dim, v_dim, dt, _stream()))
+        _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, num_kv_heads, head_dim, v_dim, T,
+        None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), dt, _stream()))
     return out
