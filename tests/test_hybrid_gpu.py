@@ -313,17 +313,19 @@ def test_delta_rule_keeps_a_far_write_and_loses_it_with_decay():
         assert abs(float(got[-1, 0, 7]) * d ** 0.5 - want) < 1e-3
 
 
-@pytest.mark.parametrize("taps", [1, 2, 3, 5])
-def test_short_convolution_across_portions_and_reused_slots(taps):
+@pytest.mark.parametrize("taps,dtype,C", [(1, torch.float32, 70), (2, torch.float32, 70), (3, torch.float32, 70),
+                                          (5, torch.float32, 70), (2, torch.bfloat16, 72), (4, torch.bfloat16, 136),
+                                          (3, torch.bfloat16, 70), (5, torch.bfloat16, 72)])
+def test_short_convolution_across_portions_and_reused_slots(taps, dtype, C):
+    """Scalar form (float32, odd widths, many taps) and the 8-channel form (16-bit, 2-4 taps)."""
     from mi355_decode import ops
     g = torch.Generator().manual_seed(taps)
-    C = 70
-    w = torch.randn(C, taps, generator=g)
-    state = torch.full((3, max(taps - 1, 1), C), float("nan"), device="cuda")[:, : taps - 1]
-    state = state.contiguous() if taps > 1 else torch.zeros(3, 0, C, device="cuda")
+    w = torch.randn(C, taps, generator=g).to(dtype)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    state = torch.full((3, taps - 1, C), float("nan"), device="cuda") if taps > 1 else torch.zeros(3, 0, C, device="cuda")
     for T, slot in ((23, 1), (9, 1), (40, 0)):                     # slot 1 is used twice: its old state must not leak
-        x = torch.randn(T, C + 8, generator=g)[:, 8:]
-        ref = R.short_conv_silu(x, w)
+        x = torch.randn(T, C + 8, generator=g).to(dtype)[:, 8:]
+        ref = R.short_conv_silu(x.float(), w.float())
         for cuts in ([T], [1] * T, [2, 1, 3] + [T - 6]):
             outs, at = [], 0
             for n in cuts:
@@ -331,9 +333,9 @@ def test_short_convolution_across_portions_and_reused_slots(taps):
                 outs.append(ops.causal_conv_silu(xs, w.cuda(), state, torch.zeros(n, dtype=torch.int32, device="cuda"),
                                                  torch.arange(at, at + n, dtype=torch.int64, device="cuda"),
                                                  torch.tensor([0, n], dtype=torch.int32, device="cuda"),
-                                                 torch.tensor([slot], dtype=torch.int32, device="cuda")).cpu())
+                                                 torch.tensor([slot], dtype=torch.int32, device="cuda")).float().cpu())
                 at += n
-            assert (torch.cat(outs) - ref).abs().max() <= 1e-5 * ref.abs().max(), (T, cuts)
+            assert (torch.cat(outs) - ref).abs().max() <= tol * ref.abs().max(), (T, cuts)
 
 
 # ------------------------------------------------------------------------------------------ #

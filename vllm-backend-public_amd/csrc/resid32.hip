@@ -93,8 +93,30 @@ __global__ __launch_bounds__(256) void rms_norm_mix_f32_kernel(float* __restrict
   }
 }
 
+// 0.5 z (1 + tanh(w)) = z / (1 + exp(-2 w)), w = sqrt(2 / pi) (z + 0.044715 z^3)
 __device__ __forceinline__ float gelu_tanh_f(float z) {
-  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z / (1.0f + expf(-1.5957691216057308f * (z + 0.044715f * z * z * z)));
+}
+
+// 16-bit rows, 8 elements per thread (16-byte loads and stores)
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_tanh_and_mul_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x,
+                                                                    int64_t x_stride, int64_t num_tokens, int inter) {
+  const int vec_per_row = inter >> 3;
+  const int64_t total = num_tokens * vec_per_row;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t row = i / vec_per_row;
+    const int v = static_cast<int>(i % vec_per_row);
+    const uint16_t* xr = x + row * x_stride;
+    float g[8], u[8], y[8];
+    unpack8<T>(MI355_LD(uint4, x, xr + 8 * v), g);
+    unpack8<T>(MI355_LD(uint4, x, xr + inter + 8 * v), u);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      y[j] = g[j] * __frcp_rn(1.0f + __expf(-1.5957691216057308f * (g[j] + 0.044715f * g[j] * g[j] * g[j]))) * u[j];
+    MI355_ST(uint4, out, out + row * inter + 8 * v, pack8<T>(y));
+  }
 }
 
 template <typename T>
@@ -224,6 +246,16 @@ extern "C" int32_t mi355_gelu_tanh_and_mul(void* out, const void* x, int64_t x_s
   REQ_DTYPE(dtype);
   if (num_tokens == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype != MI355_F32 && inter % 8 == 0 && x_stride % 8 == 0 && aligned16(x) && aligned16(out)) {
+    const dim3 grid = stride_grid(num_tokens * (inter / 8));
+    if (dtype == MI355_BF16)
+      hipLaunchKernelGGL((gelu_tanh_and_mul_vec_kernel<BF16>), grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
+                         static_cast<const uint16_t*>(x), x_stride, num_tokens, inter);
+    else
+      hipLaunchKernelGGL((gelu_tanh_and_mul_vec_kernel<F16>), grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
+                         static_cast<const uint16_t*>(x), x_stride, num_tokens, inter);
+    return check_launch("gelu_tanh_and_mul");
+  }
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((gelu_tanh_and_mul_kernel<TT>), stride_grid(num_tokens * inter), dim3(256),
                                                   0, s, static_cast<Elem<TT>::S*>(out),
                                                   static_cast<const Elem<TT>::S*>(x), x_stride, num_tokens, inter));

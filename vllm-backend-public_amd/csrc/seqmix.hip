@@ -273,6 +273,49 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
   }
 }
 
+// 16-bit rows, 8 channels per thread, the taps a template constant
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void causal_conv_silu_vec_kernel(
+    uint16_t* __restrict__ y, const uint16_t* __restrict__ x, int64_t x_stride, const uint16_t* __restrict__ w,
+    const float* __restrict__ state, const int32_t* __restrict__ tok_seq, const int64_t* __restrict__ positions,
+    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, int64_t num_tokens, int C) {
+  const int vec_per_row = C >> 3;
+  const int64_t total = num_tokens * vec_per_row;
+  for (int64_t idx = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; idx < total;
+       idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = idx / vec_per_row;
+    const int c8 = static_cast<int>(idx % vec_per_row) * 8;
+    const int s = MI355_LD(int32_t, tok_seq, tok_seq + t);
+    const int64_t cs = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s);
+    const int64_t p = MI355_LD(int64_t, positions, positions + t);
+    const float* st = state + static_cast<int64_t>(MI355_LD(int32_t, state_slots, state_slots + s)) * (TAPS - 1) * C;
+    float wv[TAPS][8];                                  // weights of the 8 channels: 8 * TAPS contiguous values
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) unpack8<T>(MI355_LD(uint4, w, w + static_cast<int64_t>(c8) * TAPS + 8 * j), wv[j]);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < TAPS; ++j) {
+      const int back = TAPS - 1 - j;
+      if (p - back < 0) continue;
+      const int64_t src = t - back;
+      float xv[8];
+      if (src >= cs) {
+        unpack8<T>(MI355_LD(uint4, x, x + src * x_stride + c8), xv);
+      } else {
+        const float* sr = st + (src - cs + TAPS - 1) * C + c8;
+        const float4 a = MI355_LD(float4, state, sr), b = MI355_LD(float4, state, sr + 4);
+        xv[0] = a.x, xv[1] = a.y, xv[2] = a.z, xv[3] = a.w, xv[4] = b.x, xv[5] = b.y, xv[6] = b.z, xv[7] = b.w;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += (&wv[0][0])[i * TAPS + j] * xv[i];
+    }
+    float o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = acc[i] / (1.0f + expf(-acc[i]));
+    MI355_ST(uint4, y, y + t * C + c8, pack8<T>(o));
+  }
+}
+
 constexpr int kMaxTaps = 16;
 
 template <typename T>
@@ -397,6 +440,19 @@ __global__ __launch_bounds__(64) void gated_delta_rule_kernel(
 // The loop then reads the next token's rows while it works on the current one.
 constexpr int kSplit = 8;
 
+// sum over the 8 adjacent lanes of a group, in every lane of it, by data-parallel-primitive moves
+// (no trip through the LDS crossbar): swap within pairs, swap pairs within quads, mirror the half row
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float sum8(float v) {
+  v += dpp_move<0xB1>(v);       // quad_perm [1, 0, 3, 2]
+  v += dpp_move<0x4E>(v);       // quad_perm [2, 3, 0, 1]
+  v += dpp_move<0x141>(v);      // row_half_mirror: lane i of 8 takes lane 7 - i
+  return v;
+}
+
 template <typename T>
 __global__ __launch_bounds__(64) void delta_prep_kernel(
     float* __restrict__ kq, float* __restrict__ dec, float* __restrict__ bet, const typename Elem<T>::S* __restrict__ qkv,
@@ -462,10 +518,13 @@ __global__ __launch_bounds__(64) void gated_delta_rule_split_kernel(
     const int i = r * DR + j;
     S[j] = (live && !fresh && i < d) ? MI355_LD(float, state, sp + static_cast<int64_t>(i) * dv + col) : 0.f;
   }
-  // the rows of the next PF tokens travel while the current PF tokens are worked on: a token's
-  // arithmetic is far shorter than a trip to memory
-  float nk[PF][DR], nq[PF][DR], na[PF][DR], nb[PF], nv[PF];
-  auto fetch = [&](int64_t first) {
+  // Two register sets of PF tokens each: while one is worked on, the rows of the PF tokens after
+  // it travel into the other (a token's arithmetic is far shorter than a trip to memory).
+  struct Rows {
+    float k[PF][DR], q[PF][DR], a[PF][DR], b[PF], v[PF];
+  };
+  Rows A, B;
+  auto fetch = [&](Rows& w, int64_t first) {
 #pragma unroll
     for (int u = 0; u < PF; ++u) {
       int64_t t = first + u;
@@ -475,54 +534,47 @@ __global__ __launch_bounds__(64) void gated_delta_rule_split_kernel(
 #pragma unroll
       for (int j = 0; j < DR; j += 4) {
         const float4 a4 = MI355_LD(float4, kq, kp + j), b4 = MI355_LD(float4, kq, kp + dp + j), c4 = MI355_LD(float4, dec, ap + j);
-        nk[u][j] = a4.x, nk[u][j + 1] = a4.y, nk[u][j + 2] = a4.z, nk[u][j + 3] = a4.w;
-        nq[u][j] = b4.x, nq[u][j + 1] = b4.y, nq[u][j + 2] = b4.z, nq[u][j + 3] = b4.w;
-        na[u][j] = c4.x, na[u][j + 1] = c4.y, na[u][j + 2] = c4.z, na[u][j + 3] = c4.w;
+        w.k[u][j] = a4.x, w.k[u][j + 1] = a4.y, w.k[u][j + 2] = a4.z, w.k[u][j + 3] = a4.w;
+        w.q[u][j] = b4.x, w.q[u][j + 1] = b4.y, w.q[u][j + 2] = b4.z, w.q[u][j + 3] = b4.w;
+        w.a[u][j] = c4.x, w.a[u][j + 1] = c4.y, w.a[u][j + 2] = c4.z, w.a[u][j + 3] = c4.w;
       }
-      nb[u] = MI355_LD(float, bet, bet + t * H + h);
-      nv[u] = live ? MI355_LDF(T, qkv, qkv + t * stride + v_off + h * dv + col) : 0.f;
+      w.b[u] = MI355_LD(float, bet, bet + t * H + h);
+      w.v[u] = live ? MI355_LDF(T, qkv, qkv + t * stride + v_off + h * dv + col) : 0.f;
     }
   };
-  fetch(cs);
-  for (int64_t i0 = 0; i0 < n; i0 += PF) {
-    float k[PF][DR], q[PF][DR], a[PF][DR], b[PF], vj[PF];
-#pragma unroll
-    for (int u = 0; u < PF; ++u) {
-#pragma unroll
-      for (int j = 0; j < DR; ++j) k[u][j] = nk[u][j], q[u][j] = nq[u][j], a[u][j] = na[u][j];
-      b[u] = nb[u], vj[u] = nv[u];
-    }
-    if (i0 + PF < n) fetch(cs + i0 + PF);
+  auto work = [&](const Rows& w, int64_t i0) {
 #pragma unroll
     for (int u = 0; u < PF; ++u) {
       if (i0 + u >= n) break;
       float d0 = 0.f, d1 = 0.f;
 #pragma unroll
       for (int j = 0; j < DR; j += 2) {
-        S[j] *= a[u][j];
-        S[j + 1] *= a[u][j + 1];
-        d0 += S[j] * k[u][j];
-        d1 += S[j + 1] * k[u][j + 1];
+        S[j] *= w.a[u][j];
+        S[j + 1] *= w.a[u][j + 1];
+        d0 += S[j] * w.k[u][j];
+        d1 += S[j + 1] * w.k[u][j + 1];
       }
-      float dot = d0 + d1;
-      dot += __shfl_xor(dot, 1, 64);
-      dot += __shfl_xor(dot, 2, 64);
-      dot += __shfl_xor(dot, 4, 64);
-      const float uu = b[u] * (vj[u] - dot);
+      const float dot = sum8(d0 + d1);
+      const float uu = w.b[u] * (w.v[u] - dot);
       float o0 = 0.f, o1 = 0.f;
 #pragma unroll
       for (int j = 0; j < DR; j += 2) {
-        S[j] += k[u][j] * uu;
-        S[j + 1] += k[u][j + 1] * uu;
-        o0 += S[j] * q[u][j];
-        o1 += S[j + 1] * q[u][j + 1];
+        S[j] += w.k[u][j] * uu;
+        S[j + 1] += w.k[u][j + 1] * uu;
+        o0 += S[j] * w.q[u][j];
+        o1 += S[j + 1] * w.q[u][j + 1];
       }
-      float out = o0 + o1;
-      out += __shfl_xor(out, 1, 64);
-      out += __shfl_xor(out, 2, 64);
-      out += __shfl_xor(out, 4, 64);
+      const float out = sum8(o0 + o1);
       if (live && r == 0) MI355_ST(float, o, o + ((cs + i0 + u) * H + h) * dv + col, out);
     }
+  };
+  fetch(A, cs);
+  for (int64_t i0 = 0; i0 < n; i0 += 2 * PF) {
+    if (i0 + PF < n) fetch(B, cs + i0 + PF);
+    work(A, i0);
+    if (i0 + PF >= n) break;
+    if (i0 + 2 * PF < n) fetch(A, cs + i0 + 2 * PF);
+    work(B, i0 + PF);
   }
   if (live) {
 #pragma unroll
@@ -664,6 +716,22 @@ extern "C" int32_t mi355_causal_conv_silu(void* y, const void* x, int64_t x_stri
   REQ_DTYPE(dtype);
   if (num_tokens == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype != MI355_F32 && taps >= 2 && taps <= 4 && channels % 8 == 0 && x_stride % 8 == 0 && aligned16(x) &&
+      aligned16(y) && aligned16(weight) && aligned16(state)) {
+    const int64_t vecs = num_tokens * (channels / 8);
+    const dim3 vgrid(static_cast<unsigned>((vecs + 255) / 256 > 65536 ? 65536 : (vecs + 255) / 256));
+#define MI355_CONV(TT, TAPS)                                                                                      \
+  hipLaunchKernelGGL((causal_conv_silu_vec_kernel<TT, TAPS>), vgrid, dim3(256), 0, s, static_cast<uint16_t*>(y),  \
+                     static_cast<const uint16_t*>(x), x_stride, static_cast<const uint16_t*>(weight), state,     \
+                     tok_seq, positions, cu_seqlens, state_slots, num_tokens, channels)
+    if (dtype == MI355_BF16) {
+      if (taps == 2) MI355_CONV(BF16, 2); else if (taps == 3) MI355_CONV(BF16, 3); else MI355_CONV(BF16, 4);
+    } else {
+      if (taps == 2) MI355_CONV(F16, 2); else if (taps == 3) MI355_CONV(F16, 3); else MI355_CONV(F16, 4);
+    }
+#undef MI355_CONV
+    return check_launch("causal_conv_silu");
+  }
   const dim3 grid(static_cast<unsigned>(num_tokens), static_cast<unsigned>((channels + 255) / 256 > 64 ? 64 : (channels + 255) / 256));
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((causal_conv_silu_kernel<TT>), grid, dim3(256), 0, s,
                                                   static_cast<Elem<TT>::S*>(y), static_cast<const Elem<TT>::S*>(x),
@@ -745,7 +813,7 @@ extern "C" int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t str
     const dim3 pgrid(static_cast<unsigned>(num_tokens), static_cast<unsigned>(num_kv_heads + num_heads));
     const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>((v_dim + 7) / 8));
 #define MI355_DSPLIT(TT, DR)                                                                                          \
-  hipLaunchKernelGGL((gated_delta_rule_split_kernel<TT, DR, (DR <= 16 ? 4 : 2)>), grid, dim3(64), 0, s, o,            \
+  hipLaunchKernelGGL((gated_delta_rule_split_kernel<TT, DR, (DR <= 8 ? 4 : DR <= 16 ? 2 : 1)>), grid, dim3(64), 0, s, o,            \
                      static_cast<const Elem<TT>::S*>(qkv), stride, v_off, kq, dec, bet, state, cu_seqlens, positions, \
                      state_slots, num_heads, num_kv_heads, head_dim, v_dim)
     MI355_DISPATCH_DTYPE3(dtype, {

@@ -170,9 +170,9 @@ def kernel_table(width: int, prompt_len: int, batch: int) -> list:
     od = torch.empty(batch, H * dv, device=dev, dtype=bf)
     ws = torch.empty(max(ops.decode_workspace_bytes(batch, H, d, 16), 16), dtype=torch.uint8, device=dev)
     dtiles = torch.stack([seqd, seqd, torch.ones_like(seqd)], dim=1).contiguous()
-    part = torch.empty(8 * batch * H * dv, device=dev)
+    part = torch.empty(16 * batch * H * dv, device=dev)
     t_h = _time(lambda: ops.sigmoid_window_attn(qd, kc, vct, bt, seqd, posd, temp, bias, gd, H, window, d ** -0.5, out=od,
-                                                tiles=dtiles, partial=part, num_splits=8))
+                                                tiles=dtiles, partial=part, num_splits=16))
     t_l = _time(lambda: ops.paged_attn_decode(qd, kc, vct, bt, ctxd, H, G, d, d ** -0.5, num_splits=4, workspace=ws, out=od))
     row("sigmoid_window_attn", f"decode {batch} rows at context {P}, window {window}", t_h, "hbm",
         batch * min(P, window) * G * (d + dv) * 2, "paged_attn_decode (whole context)", t_l, batch * P * G * 2 * d * 2)

@@ -188,14 +188,14 @@ class HybridRunner(ModelRunner):
             self._rotary[key] = rotary_table(rot_dims, base, self.max_blocks * BLOCK_SIZE, self.device)
         return self._rotary[key]
 
-    MAX_KEY_SPLITS = 8
+    MAX_KEY_SPLITS = 16
 
     def key_splits(self, b: StepBatch, a) -> dict:
         """Workgroups per tile for the window attention: more than one only for batches of few rows
         (decoded tokens), where one workgroup per row and kv head would leave most of the chip idle."""
         if b.tiles is None or b.long_chunks or b.num_tokens > self.max_num_seqs:
             return {}
-        n = min(self.MAX_KEY_SPLITS, max(a.window // 64, 1))
+        n = min(self.MAX_KEY_SPLITS, max(a.window // 64, 1), max(2048 // max(b.num_tokens * a.kv_heads, 1), 1))
         return {"partial": self._attn_partial, "num_splits": n} if n > 1 else {}
 
     def kv_cache_bytes_per_block(self) -> int:
