@@ -131,27 +131,31 @@ __global__ __launch_bounds__(64) void sigmoid_window_attn_kernel(
   }
 }
 
-// The matrix-core form for 16-bit activations, d a multiple of 32, dv a multiple of 16.  One
-// workgroup per (tile of up to 16 consecutive rows of one chunk, kv head); its waves take the
-// query heads of the group, so the K / V fragments they all read stay in the CU's cache.  Keys are
+// The matrix-core form for 16-bit activations, d a multiple of 32, dv a multiple of 16.  One wave
+// per (tile of up to 16 consecutive rows of one chunk, block of HB query heads of one kv head): the
+// K and V fragments it loads serve all HB heads, whose query fragments and accumulators stay in
+// registers (a wave per head would pull the same pages through the cache HB times).  Keys are
 // taken 32 at a time (two pages).  Scores are computed transposed, S^T = K Q^T, so that a lane ends
 // up holding, for its query (lane % 16), eight weights -- keys 4 (lane / 16) + r of either page --
 // which is exactly an A-operand fragment of the P V product once V's fragment lists the same
 // eight keys: with V pages stored [dv, 16 tokens] that is two 8-byte loads.  Scores, the sigmoid
 // and the accumulators are fp32; the weights are rounded to the storage type for the second product.
-template <typename T>
-__global__ __launch_bounds__(512) void sigmoid_window_attn_mfma_kernel(
+// gridDim.z > 1: the key tiles are dealt out to the z blocks in turn and each writes its fp32 sums
+// (no gate) to its slab of `partial`; the weights are not normalised, so the slabs simply add up.
+template <typename T, int HB, int DS, int CB>
+__global__ __launch_bounds__(256) void sigmoid_window_attn_mfma_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ tiles, const int64_t* __restrict__ positions, const float* __restrict__ temp,
-    const float* __restrict__ bias, const uint16_t* __restrict__ gate, int64_t gate_stride, int H, int G, int d, int dv,
-    int window, float scale, float* __restrict__ partial, int64_t partial_stride) {
-  constexpr int kMaxD = 256 / 32, kMaxDV = 256 / 16;
-  // gridDim.z > 1: the key tiles are dealt out to the z blocks in turn and each writes its fp32 sums
-  // (no gate) to its slab of `partial`; the weights are not normalised, so the slabs simply add up
+    const int32_t* __restrict__ tiles, int num_tiles, const int64_t* __restrict__ positions,
+    const float* __restrict__ temp, const float* __restrict__ bias, const uint16_t* __restrict__ gate,
+    int64_t gate_stride, int H, int G, int d, int dv, int window, float scale, float* __restrict__ partial,
+    int64_t partial_stride) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int tile = blockIdx.x * (blockDim.x >> 6) + wave;
+  if (tile >= num_tiles) return;                        // (no workgroup barrier below)
+  const int rep = H / G, hbs = rep / HB;
+  const int g = blockIdx.y / hbs, h0 = g * rep + (blockIdx.y % hbs) * HB;
   const int nz = gridDim.z, z = blockIdx.z;
-  const int tile = blockIdx.x, g = blockIdx.y, rep = H / G;
-  const int wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6, lane = threadIdx.x & 63;
   const int li = lane & 15, kk = lane >> 4;
   const int seq = MI355_LD(int32_t, tiles, tiles + 3 * tile);
   const int64_t row0 = MI355_LD(int32_t, tiles, tiles + 3 * tile + 1);
@@ -162,86 +166,109 @@ __global__ __launch_bounds__(512) void sigmoid_window_attn_mfma_kernel(
   const int64_t p_last = p0 + nrows - 1;
   int64_t lo = p0 - window + 1;
   if (lo < 0) lo = 0;
-  const int64_t my_p = p0 + li;                       // position of this lane's query (rows past nrows: masked out)
-  for (int hh = wave; hh < rep; hh += nwaves) {
-    const int h = g * rep + hh;
-    uint4 qf[kMaxD];
+  const int64_t my_p = p0 + li;                         // position of this lane's query (rows past nrows: masked out)
+  uint4 qf[HB][DS];
+  float mul[HB], add[HB];
+  f32x4 acc[HB][CB];
 #pragma unroll
-    for (int s = 0; s < kMaxD; ++s) {
-      qf[s] = make_uint4(0, 0, 0, 0);
+  for (int i = 0; i < HB; ++i) {
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+      qf[i][s] = make_uint4(0, 0, 0, 0);
       if (s < ds && li < nrows)
-        qf[s] = MI355_LD(uint4, q, q + (row0 + li) * q_stride + static_cast<int64_t>(h) * d + 32 * s + 8 * kk);
+        qf[i][s] = MI355_LD(uint4, q, q + (row0 + li) * q_stride + static_cast<int64_t>(h0 + i) * d + 32 * s + 8 * kk);
     }
-    const float mul = scale * MI355_LD(float, temp, temp + h), add = MI355_LD(float, bias, bias + h);
-    f32x4 acc[kMaxDV];
+    mul[i] = -1.4426950408889634f * scale * MI355_LD(float, temp, temp + h0 + i);
+    add[i] = -1.4426950408889634f * MI355_LD(float, bias, bias + h0 + i);
 #pragma unroll
-    for (int c = 0; c < kMaxDV; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int64_t base = ((lo >> 5) << 5) + 32 * z; base <= p_last; base += 32 * nz) {
-      uint32_t pw[4];                                   // 8 weights of this lane's query, packed
-      int64_t pages[2];
+    for (int c = 0; c < CB; ++c) acc[i][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  for (int64_t base = ((lo >> 5) << 5) + 32 * z; base <= p_last; base += 32 * nz) {
+    // every load of the tile is issued before the first product: one trip to memory per tile, not
+    // one per fragment
+    uint4 kf[2][DS];
+    uint2 vf[2][CB];
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int64_t kb = base + 16 * half;
+    for (int half = 0; half < 2; ++half) {
+      const int64_t kb = base + 16 * half;
+      const bool have = kb <= p_last;
+      const int64_t page = have ? MI355_LD(int32_t, block_tables, bt + kb / kPage) : 0;
+      const uint16_t* kr = k_cache + ((page * G + g) * kPage + li) * d + 8 * kk;
+      const uint16_t* vr = v_cache + ((page * G + g) * dv + li) * kPage + 4 * kk;
+#pragma unroll
+      for (int s = 0; s < DS; ++s)
+        kf[half][s] = (have && s < ds) ? MI355_LD(uint4, k_cache, kr + 32 * s) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int c = 0; c < CB; ++c)
+        vf[half][c] = (have && c < cbs) ? MI355_LD(uint2, v_cache, vr + 16 * c * kPage) : make_uint2(0, 0);
+    }
+    uint32_t pw[HB][4];                                 // 8 weights of this lane's query per head, packed
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int64_t kb = base + 16 * half;
+      bool vis[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int64_t key = kb + 4 * kk + r;
+        vis[r] = li < nrows && key <= my_p && my_p - key < window;
+      }
+#pragma unroll
+      for (int i = 0; i < HB; ++i) {
         f32x4 sacc = f32x4{0.f, 0.f, 0.f, 0.f};
-        pages[half] = -1;
-        if (kb <= p_last) {
-          pages[half] = MI355_LD(int32_t, block_tables, bt + kb / kPage);
-          const uint16_t* kr = k_cache + ((pages[half] * G + g) * kPage + li) * d + 8 * kk;
 #pragma unroll
-          for (int s = 0; s < kMaxD; ++s)
-            if (s < ds) sacc = T::mfma(MI355_LD(uint4, k_cache, kr + 32 * s), qf[s], sacc);
-        }
+        for (int s = 0; s < DS; ++s)
+          if (s < ds) sacc = T::mfma(kf[half][s], qf[i][s], sacc);
         float w[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int64_t key = kb + 4 * kk + r;
-          const bool vis = li < nrows && key <= my_p && my_p - key < window;
-          w[r] = vis ? __frcp_rn(1.0f + __expf(-(sacc[r] * mul + add))) : 0.f;
-        }
-        pw[2 * half] = T::pack2(w[0], w[1]);
-        pw[2 * half + 1] = T::pack2(w[2], w[3]);
+        for (int r = 0; r < 4; ++r)                       // sigmoid(x) = 1 / (1 + 2^(-x log2 e))
+          w[r] = vis[r] ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(sacc[r] * mul[i] + add[i])) : 0.f;
+        pw[i][2 * half] = T::pack2(w[0], w[1]);
+        pw[i][2 * half + 1] = T::pack2(w[2], w[3]);
       }
-      const uint4 pf = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+    }
+    if (base + 31 > p_last) {
+      // slots past the newest key may hold anything (0 * NaN is NaN): clear them in the last tile
 #pragma unroll
-      for (int c = 0; c < kMaxDV; ++c) {
-        if (c < cbs) {
-          uint2 v0 = make_uint2(0, 0), v1 = make_uint2(0, 0);
-          if (pages[0] >= 0)
-            v0 = MI355_LD(uint2, v_cache, v_cache + ((pages[0] * G + g) * dv + 16 * c + li) * kPage + 4 * kk);
-          if (pages[1] >= 0)
-            v1 = MI355_LD(uint2, v_cache, v_cache + ((pages[1] * G + g) * dv + 16 * c + li) * kPage + 4 * kk);
-          // slots past the newest key may hold anything (0 * NaN is NaN): clear them in the last tile
-          if (base + 31 > p_last) {
+      for (int half = 0; half < 2; ++half) {
+        const int64_t k0 = base + 16 * half + 4 * kk;
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
-              uint2& vv = half == 0 ? v0 : v1;
-              const int64_t k0 = base + 16 * half + 4 * kk;
-              if (k0 > p_last) vv.x &= 0xFFFF0000u;
-              if (k0 + 1 > p_last) vv.x &= 0x0000FFFFu;
-              if (k0 + 2 > p_last) vv.y &= 0xFFFF0000u;
-              if (k0 + 3 > p_last) vv.y &= 0x0000FFFFu;
-            }
-          }
-          acc[c] = T::mfma(pf, make_uint4(v0.x, v0.y, v1.x, v1.y), acc[c]);
+        for (int c = 0; c < CB; ++c) {
+          if (k0 > p_last) vf[half][c].x &= 0xFFFF0000u;
+          if (k0 + 1 > p_last) vf[half][c].x &= 0x0000FFFFu;
+          if (k0 + 2 > p_last) vf[half][c].y &= 0xFFFF0000u;
+          if (k0 + 3 > p_last) vf[half][c].y &= 0x0000FFFFu;
         }
       }
     }
-    // C layout: this lane holds rows 4 kk + r of column li of every 16-column block
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+      if (c < cbs) {
+        const uint4 v4 = make_uint4(vf[0][c].x, vf[0][c].y, vf[1][c].x, vf[1][c].y);
+#pragma unroll
+        for (int i = 0; i < HB; ++i)
+          acc[i][c] = T::mfma(make_uint4(pw[i][0], pw[i][1], pw[i][2], pw[i][3]), v4, acc[i][c]);
+      }
+    }
+  }
+  // C layout: this lane holds rows 4 kk + r of column li of every 16-column block
+#pragma unroll
+  for (int i = 0; i < HB; ++i) {
+    const int h = h0 + i;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int rr = 4 * kk + r;
       if (rr >= nrows) continue;
       if (partial != nullptr) {
 #pragma unroll
-        for (int c = 0; c < kMaxDV; ++c)
-          if (c < cbs) MI355_ST(float, partial, partial + z * partial_stride + ((row0 + rr) * H + h) * dv + 16 * c + li, acc[c][r]);
+        for (int c = 0; c < CB; ++c)
+          if (c < cbs) MI355_ST(float, partial, partial + z * partial_stride + ((row0 + rr) * H + h) * dv + 16 * c + li, acc[i][c][r]);
         continue;
       }
       float gt = 1.0f;
       if (gate != nullptr) gt = 1.0f / (1.0f + expf(-T::to_f(MI355_LD(uint16_t, gate, gate + (row0 + rr) * gate_stride + h))));
 #pragma unroll
-      for (int c = 0; c < kMaxDV; ++c)
-        if (c < cbs) MI355_ST(uint16_t, out, out + ((row0 + rr) * H + h) * dv + 16 * c + li, T::from_f(acc[c][r] * gt));
+      for (int c = 0; c < CB; ++c)
+        if (c < cbs) MI355_ST(uint16_t, out, out + ((row0 + rr) * H + h) * dv + 16 * c + li, T::from_f(acc[i][c][r] * gt));
     }
   }
 }
@@ -682,20 +709,34 @@ extern "C" int32_t mi355_sigmoid_window_attn(void* out, const void* q, int64_t q
     const int rep = num_heads / num_kv_heads;
     const bool split = partial != nullptr && num_splits > 1;
     MI355_REQUIRE(num_splits >= 0 && num_splits <= 64, MI355_ERR_INVALID, "sigmoid_window_attn: %d key splits", num_splits);
-    const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(num_kv_heads), split ? num_splits : 1);
-    const dim3 block(64u * static_cast<unsigned>(rep < 8 ? rep : 8));
+    const bool small = head_dim <= 128 && v_dim <= 128;
+    const int hb = !small ? 1 : (rep % 4 == 0 ? 4 : rep % 2 == 0 ? 2 : 1);      // query heads per wave
+    const int waves = num_tiles < 4 ? num_tiles : 4;                              // a tile per wave
+    const dim3 grid(static_cast<unsigned>((num_tiles + waves - 1) / waves), static_cast<unsigned>(num_kv_heads * (rep / hb)),
+                    split ? num_splits : 1);
+    const dim3 block(64u * static_cast<unsigned>(waves));
     const int64_t slab = num_tokens * num_heads * v_dim;
-#define MI355_WMFMA(TT)                                                                                             \
-  hipLaunchKernelGGL((sigmoid_window_attn_mfma_kernel<TT>), grid, block, 0, s, static_cast<uint16_t*>(out),          \
-                     static_cast<const uint16_t*>(q), q_stride, static_cast<const uint16_t*>(k_cache),               \
-                     static_cast<const uint16_t*>(v_cache), block_tables, max_blocks, tiles, positions, temp, bias,  \
-                     static_cast<const uint16_t*>(gate), gate_stride, num_heads, num_kv_heads, head_dim, v_dim,      \
-                     window, scale, split ? partial : nullptr, slab);                                                \
-  if (split)                                                                                                        \
-    hipLaunchKernelGGL((window_attn_reduce_kernel<TT>), dim3(static_cast<unsigned>((slab + 255) / 256 > 4096 ? 4096 : (slab + 255) / 256)), \
-                       dim3(256), 0, s, static_cast<uint16_t*>(out), partial, static_cast<const uint16_t*>(gate),    \
-                       gate_stride, num_tokens, num_heads, v_dim, num_splits)
-    if (dtype == MI355_BF16) { MI355_WMFMA(BF16); } else { MI355_WMFMA(F16); }
+#define MI355_WMFMA(TT, HB, DS, CB)                                                                                 \
+  hipLaunchKernelGGL((sigmoid_window_attn_mfma_kernel<TT, HB, DS, CB>), grid, block, 0, s,                          \
+                     static_cast<uint16_t*>(out), static_cast<const uint16_t*>(q), q_stride,                        \
+                     static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(v_cache), block_tables,    \
+                     max_blocks, tiles, num_tiles, positions, temp, bias, static_cast<const uint16_t*>(gate),       \
+                     gate_stride, num_heads, num_kv_heads, head_dim, v_dim, window, scale,                          \
+                     split ? partial : nullptr, slab)
+#define MI355_WMFMA_HB(TT)                                                                                          \
+  do {                                                                                                              \
+    if (!small) MI355_WMFMA(TT, 1, 8, 16);                                                                          \
+    else if (hb == 4) MI355_WMFMA(TT, 4, 4, 8);                                                                     \
+    else if (hb == 2) MI355_WMFMA(TT, 2, 4, 8);                                                                     \
+    else MI355_WMFMA(TT, 1, 4, 8);                                                                                  \
+    if (split)                                                                                                      \
+      hipLaunchKernelGGL((window_attn_reduce_kernel<TT>),                                                           \
+                         dim3(static_cast<unsigned>((slab + 255) / 256 > 4096 ? 4096 : (slab + 255) / 256)),        \
+                         dim3(256), 0, s, static_cast<uint16_t*>(out), partial, static_cast<const uint16_t*>(gate), \
+                         gate_stride, num_tokens, num_heads, v_dim, num_splits);                                    \
+  } while (0)
+    if (dtype == MI355_BF16) MI355_WMFMA_HB(BF16); else MI355_WMFMA_HB(F16);
+#undef MI355_WMFMA_HB
 #undef MI355_WMFMA
     return check_launch("sigmoid_window_attn (matrix cores)");
   }

@@ -158,8 +158,10 @@ def kernel_table(width: int, prompt_len: int, batch: int) -> list:
     o = torch.empty(P, H * dv, device=dev, dtype=bf)
     keys = sum(min(i + 1, window) for i in range(P))
     tiles = torch.from_numpy(ops.query_tiles([0, P])).to(dev)
+    nsp = max(min(16, 2048 // max(tiles.shape[0] * G * max(H // G // 4, 1), 1)), 1)
+    ppart = torch.empty(nsp * P * H * dv, device=dev)
     t_h = _time(lambda: ops.sigmoid_window_attn(q, kc, vct, bt[:1], seq0, pos, temp, bias, gate, H, window, d ** -0.5, out=o,
-                                                tiles=tiles), 5)
+                                                tiles=tiles, partial=ppart, num_splits=nsp), 5)
     t_l = _time(lambda: ops.paged_attn_prefill(q, kc, vct, bt[:1], cu, ctx, P, H, G, d, d ** -0.5, out=o), 5)
     row("sigmoid_window_attn", f"prefill {P} tokens, window {window}, {H}/{G} heads x {d}", t_h, "mfma", 2.0 * keys * H * (d + dv),
         "paged_attn_prefill (causal softmax)", t_l, 2.0 * (P * (P + 1) // 2) * H * 2 * d)

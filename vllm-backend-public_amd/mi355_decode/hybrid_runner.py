@@ -191,12 +191,18 @@ class HybridRunner(ModelRunner):
     MAX_KEY_SPLITS = 16
 
     def key_splits(self, b: StepBatch, a) -> dict:
-        """Workgroups per tile for the window attention: more than one only for batches of few rows
-        (decoded tokens), where one workgroup per row and kv head would leave most of the chip idle."""
-        if b.tiles is None or b.long_chunks or b.num_tokens > self.max_num_seqs:
+        """Workgroups per tile for the window attention: more than one where one wave per (tile, block
+        of heads) would leave most of the chip idle -- decoded tokens, and short or single prompts."""
+        if b.tiles is None or self.dtype == torch.float32:
             return {}
-        n = min(self.MAX_KEY_SPLITS, max(a.window // 64, 1), max(2048 // max(b.num_tokens * a.kv_heads, 1), 1))
-        return {"partial": self._attn_partial, "num_splits": n} if n > 1 else {}
+        waves = int(b.tiles.shape[0]) * a.kv_heads * max((a.heads // a.kv_heads) // 4, 1)
+        n = min(self.MAX_KEY_SPLITS, max(a.window // 64, 1), max(2048 // max(waves, 1), 1))
+        if n <= 1:
+            return {}
+        need = n * b.num_tokens * a.heads * a.vdim
+        if b.num_tokens <= self.max_num_seqs and need <= self._attn_partial.numel():
+            return {"partial": self._attn_partial, "num_splits": n}      # static: a decode graph holds its address
+        return {"partial": torch.empty(need, dtype=torch.float32, device=self.device), "num_splits": n}
 
     def kv_cache_bytes_per_block(self) -> int:
         return sum(t[0].numel() * t.element_size() for t in self.k_cache + self.v_cache)
