@@ -204,7 +204,7 @@ def test_window_attention_whole_portions_and_single_tokens(H, G, d, dv, window, 
 
 
 @pytest.mark.parametrize("H,G,d,dv,window,rot", [(4, 2, 32, 48, 20, 16), (2, 1, 128, 64, 33, 128), (8, 2, 64, 64, 200, 32),
-                                                 (16, 1, 96, 16, 7, 64)])
+                                                 (16, 1, 96, 16, 7, 64), (2, 1, 256, 256, 40, 64), (2, 2, 160, 144, 20, 32)])
 def test_window_attention_on_the_matrix_cores(H, G, d, dv, window, rot):
     """The 16-row tile form (16-bit storage) against the restatement run on the same rounded inputs:
     whole prompt, uneven portions, single rows; unused page slots hold NaN and must not leak."""
