@@ -459,13 +459,12 @@ __global__ __launch_bounds__(64) void gated_delta_rule_kernel(
 
 // ---- the gated delta rule for chunks of many tokens -------------------------------------------------
 // With one state column per lane a token costs 4 * d dependent vector operations per wave and a
-// prompt keeps only heads * dv / 64 waves busy.  Here the d rows of a column are split over R = 8
-// adjacent lanes (a wave holds 8 columns, DR = ceil(d / 8) rows each), the two dot products of a
-// token are finished with three cross-lane steps each, and everything that does not depend on the
+// prompt keeps only heads * dv / 64 waves busy.  Here the d rows of a column are split over R = 16
+// (or 8) adjacent lanes (a wave holds 64 / R columns, DR = ceil(d / R) rows each), the two dot products
+// of a token are finished with four (three) cross-lane steps each, and everything that does not depend on the
 // state -- unit-length key and query, decay, beta -- is computed for all tokens at once by
-// delta_prep_kernel, in fp32, into rows padded to 8 * DR (key / query 0, decay 1 in the padding).
+// delta_prep_kernel, in fp32, into rows padded to R * DR (key / query 0, decay 1 in the padding).
 // The loop then reads the next token's rows while it works on the current one.
-constexpr int kSplit = 8;
 
 // sum over the 8 adjacent lanes of a group, in every lane of it, by data-parallel-primitive moves
 // (no trip through the LDS crossbar): swap within pairs, swap pairs within quads, mirror the half row
@@ -473,10 +472,12 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
 }
-__device__ __forceinline__ float sum8(float v) {
+template <int R>
+__device__ __forceinline__ float sum_lanes(float v) {
   v += dpp_move<0xB1>(v);       // quad_perm [1, 0, 3, 2]
   v += dpp_move<0x4E>(v);       // quad_perm [2, 3, 0, 1]
   v += dpp_move<0x141>(v);      // row_half_mirror: lane i of 8 takes lane 7 - i
+  if (R == 16) v += dpp_move<0x128>(v);   // row_ror 8: the other half of the 16-lane row
   return v;
 }
 
@@ -522,15 +523,15 @@ __global__ __launch_bounds__(64) void delta_prep_kernel(
     MI355_ST(float, bet, bet + t * H + h, 1.0f / (1.0f + expf(-MI355_LDF(T, beta, beta + t * beta_stride + h))));
 }
 
-template <typename T, int DR, int PF>
+template <typename T, int R, int DR, int PF>
 __global__ __launch_bounds__(64) void gated_delta_rule_split_kernel(
     float* __restrict__ o, const typename Elem<T>::S* __restrict__ qkv, int64_t stride, int v_off,
     const float* __restrict__ kq, const float* __restrict__ dec, const float* __restrict__ bet, float* __restrict__ state,
     const int32_t* __restrict__ cu_seqlens, const int64_t* __restrict__ positions,
     const int32_t* __restrict__ state_slots, int H, int G, int d, int dv) {
-  constexpr int dp = kSplit * DR;
+  constexpr int dp = R * DR;
   const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int r = lane & (kSplit - 1), col = blockIdx.z * (64 / kSplit) + (lane >> 3);
+  const int r = lane & (R - 1), col = blockIdx.z * (64 / R) + lane / R;
   const int g = h / (H / G);
   const int64_t cs = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s);
   const int64_t n = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1) - cs;
@@ -581,7 +582,7 @@ __global__ __launch_bounds__(64) void gated_delta_rule_split_kernel(
         d0 += S[j] * w.k[u][j];
         d1 += S[j + 1] * w.k[u][j + 1];
       }
-      const float dot = sum8(d0 + d1);
+      const float dot = sum_lanes<R>(d0 + d1);
       const float uu = w.b[u] * (w.v[u] - dot);
       float o0 = 0.f, o1 = 0.f;
 #pragma unroll
@@ -591,7 +592,7 @@ __global__ __launch_bounds__(64) void gated_delta_rule_split_kernel(
         o0 += S[j] * w.q[u][j];
         o1 += S[j + 1] * w.q[u][j + 1];
       }
-      const float out = sum8(o0 + o1);
+      const float out = sum_lanes<R>(o0 + o1);
       if (live && r == 0) MI355_ST(float, o, o + ((cs + i0 + u) * H + h) * dv + col, out);
     }
   };
@@ -844,8 +845,9 @@ extern "C" int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t str
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (workspace != nullptr && num_tokens > 0) {
     // the form for chunks of many tokens: rows split over 8 lanes, per-token vectors prepared up front
-    const int dr = head_dim <= 32 ? 4 : head_dim <= 64 ? 8 : head_dim <= 128 ? 16 : 32;
-    const int64_t dp = 8 * dr;
+    // state rows of a column over 16 adjacent lanes (8 for heads of up to 32 rows); rows padded to dp
+    const int64_t dp = head_dim <= 32 ? 32 : head_dim <= 64 ? 64 : head_dim <= 128 ? 128 : 256;
+    const int lanes = head_dim <= 32 ? 8 : 16;
     const int64_t need = mi355_gated_delta_rule_workspace(num_tokens, num_heads, num_kv_heads, head_dim);
     MI355_REQUIRE(workspace_floats >= need && aligned16(workspace), MI355_ERR_INVALID,
                   "gated_delta_rule: workspace of %lld floats, %lld needed, 16-byte aligned",
@@ -854,9 +856,10 @@ extern "C" int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t str
     float* dec = kq + num_tokens * num_kv_heads * 2 * dp;
     float* bet = dec + num_tokens * num_heads * dp;
     const dim3 pgrid(static_cast<unsigned>(num_tokens), static_cast<unsigned>(num_kv_heads + num_heads));
-    const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>((v_dim + 7) / 8));
-#define MI355_DSPLIT(TT, DR)                                                                                          \
-  hipLaunchKernelGGL((gated_delta_rule_split_kernel<TT, DR, (DR <= 8 ? 4 : DR <= 16 ? 2 : 1)>), grid, dim3(64), 0, s, o,            \
+    const int cols = 64 / lanes;
+    const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>((v_dim + cols - 1) / cols));
+#define MI355_DSPLIT(TT, R, DR, PF)                                                                                   \
+  hipLaunchKernelGGL((gated_delta_rule_split_kernel<TT, R, DR, PF>), grid, dim3(64), 0, s, o,                         \
                      static_cast<const Elem<TT>::S*>(qkv), stride, v_off, kq, dec, bet, state, cu_seqlens, positions, \
                      state_slots, num_heads, num_kv_heads, head_dim, v_dim)
     MI355_DISPATCH_DTYPE3(dtype, {
@@ -864,8 +867,10 @@ extern "C" int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t str
                          stride, q_off, k_off, static_cast<const Elem<TT>::S*>(beta), beta_stride,
                          static_cast<const Elem<TT>::S*>(decay), decay_stride, a_log, dt_bias, per_channel, num_heads,
                          num_kv_heads, head_dim, static_cast<int>(dp));
-      if (dr == 4) MI355_DSPLIT(TT, 4); else if (dr == 8) MI355_DSPLIT(TT, 8); else if (dr == 16) MI355_DSPLIT(TT, 16);
-      else MI355_DSPLIT(TT, 32);
+      if (dp == 32) MI355_DSPLIT(TT, 8, 4, 4);
+      else if (dp == 64) MI355_DSPLIT(TT, 16, 4, 4);
+      else if (dp == 128) MI355_DSPLIT(TT, 16, 8, 4);
+      else MI355_DSPLIT(TT, 16, 16, 2);
     });
 #undef MI355_DSPLIT
     return check_launch("gated_delta_rule (split rows)");
