@@ -121,3 +121,80 @@ def test_restatement_window_edge_and_cut_invariance():
     z = R.forward(wts, cfgd, toks)
     assert torch.allclose(R.forward(wts, cfgd, toks[:17]), z[:17], atol=1e-5)     # causal
     assert float(z.abs().max()) <= 9.0
+
+
+class _StatefulRunner:
+    """A runner double whose 'model' is a running checksum per state slot and a token table in the KV
+    pages: it fails loudly when a step hands it a slot whose state does not continue the request, a
+    page that holds another request's tokens, or a chunk at position 0 that finds old state."""
+    device, V, NUM_STAGES = "cpu", 50, 1
+
+    def __init__(self, num_blocks, max_num_seqs, max_model_len, slots):
+        import numpy as np
+        self.np = np
+        self.num_blocks, self.max_num_seqs, self.num_state_slots = num_blocks, max_num_seqs, slots
+        self.max_blocks = (max_model_len + 15) // 16
+        self.pages = np.full(num_blocks * 16, -1, dtype=np.int64)
+        self.state = {s: (0, 0) for s in range(slots)}          # slot -> (tokens seen, checksum)
+        self.batches = []
+
+    def host_inputs(self, stage=0):
+        B = self.max_num_seqs
+        return self.np.zeros(3 * B, dtype=self.np.int64), self.np.zeros(B + B * self.max_blocks + B, dtype=self.np.int32)
+
+    def run_prefill(self, token_ids, positions, slot_mapping, block_tables, cu_seqlens, context_lens, max_q_len,
+                    sampling=None, logprobs=-1, prompt_logprobs=None, state_slots=None, logit_rows=None):
+        np = self.np
+        assert state_slots is not None and len(state_slots) == len(context_lens) and len(set(state_slots.tolist())) == len(state_slots)
+        self.batches.append([int(cu_seqlens[i + 1] - cu_seqlens[i]) for i in range(len(context_lens))])
+        rows = np.zeros((len(token_ids), self.V), dtype=np.float32)
+        for i, slot in enumerate(state_slots.tolist()):
+            a, b = int(cu_seqlens[i]), int(cu_seqlens[i + 1])
+            start = int(positions[a])
+            seen, acc = (0, 0) if start == 0 else self.state[slot]
+            assert seen == start, f"slot {slot} holds {seen} tokens, the chunk starts at {start}"
+            for r in range(a, b):
+                self.pages[slot_mapping[r]] = token_ids[r]
+                acc = (acc * 31 + int(token_ids[r]) + 1) % 1000003
+                p = int(positions[r])
+                ctx = self.pages[block_tables[i][np.arange(p + 1) // 16].astype(np.int64) * 16 + np.arange(p + 1) % 16]
+                rows[r, 0], rows[r, 1] = acc, int(ctx.sum())    # what the state and what the pages remember
+            self.state[slot] = (start + b - a, acc)
+        return rows[np.asarray(logit_rows, dtype=np.int64)]
+
+
+def test_forced_steps_keep_pages_and_slots_straight():
+    """LLMEngine.forced_step on a double: mixed batches, a request that sits out, requests that end
+    and hand their pages and slot to newcomers; every wanted row equals what the request alone gives."""
+    import numpy as np
+    from mi355_decode.engine import LLMEngine
+    runner = _StatefulRunner(num_blocks=12, max_num_seqs=3, max_model_len=96, slots=3)
+    eng = LLMEngine(runner, max_num_seqs=3, max_num_batched_tokens=1 << 20, max_model_len=96)
+    rng = np.random.default_rng(0)
+    toks = {r: rng.integers(0, 50, n).tolist() for r, n in (("a", 40), ("b", 17), ("c", 5), ("d", 33), ("e", 64))}
+
+    def alone(t):
+        acc, out = 0, []
+        for i, x in enumerate(t):
+            acc = (acc * 31 + x + 1) % 1000003
+            out.append((acc, sum(t[: i + 1])))
+        return out
+
+    plan = [([("a", 16), ("b", 2), ("c", 5)], ["c"]), ([("a", 1), ("d", 20)], []), ([("a", 23), ("b", 15), ("d", 1)], ["a", "b"]),
+            ([("d", 12), ("e", 64)], ["d", "e"])]
+    at = {r: 0 for r in toks}
+    for entries, end in plan:
+        req = [(r, toks[r][at[r]:at[r] + n], [0, n - 1] if n > 1 else [0]) for r, n in entries]
+        out = eng.forced_step(req, end)
+        row = 0
+        for r, t, want in req:
+            for j in want:
+                assert tuple(out[row][:2]) == tuple(float(v) for v in alone(toks[r])[at[r] + j]), (r, j)
+                row += 1
+            at[r] += len(t)
+        assert row == out.shape[0]
+    assert all(at[r] == len(toks[r]) for r in toks)
+    assert runner.batches == [[16, 2, 5], [1, 20], [23, 15, 1], [12, 64]]
+    assert eng.alloc.num_free == 12 and eng.slots.num_free == 3 and not eng.seqs
+    with pytest.raises(ValueError):
+        eng.forced_step([("z", [99], [0])])                      # outside the vocabulary
