@@ -46,6 +46,12 @@ CONFIGS = {
                         {"type": "parallel", "mixer": {"left": _left(4, 2, 32, 32, 17, 32), "right": _delta(2, 2, 32, 64, 3)},
                          "mlp": {"kind": "dense", "ff": 96}},
                         {"type": "delta", "mixer": _delta(4, 1, 64, 32, 4), "mlp": {"kind": "dense", "ff": 160}}]},
+    # a width the weight-streaming GEMM's tiled form covers (decode-sized steps in 16 bits take it)
+    "wide": {"architecture": "Lozupel", "embedding": {"scale": 1.0}, "width": 512, "vocab": 384,
+             "norm": {"eps": 1e-6}, "logit_softcap": 20.0, "loop": {"start": 0, "stop": 2, "times": 2},
+             "layers": [{"type": "parallel", "mixer": {"left": _left(8, 2, 64, 64, 24, 32), "right": _delta(4, 2, 64, 128, 4)},
+                         "mlp": {"kind": "dense", "ff": 1024}},
+                        {"type": "delta", "mixer": _delta(8, 4, 64, 64, 3), "mlp": {"kind": "dense", "ff": 512}}]},
 }
 _cache = {}
 
@@ -438,7 +444,24 @@ def test_bfloat16_tracks_the_float32_restatement():
         assert rel.max() < 0.06, rel.max()
 
 
-@pytest.mark.parametrize("name,dtype", [("loop0", "float32"), ("tail", "float32"), ("plain", "bfloat16")])
+def test_decode_sized_steps_on_the_tiled_weight_stream():
+    """bfloat16 at a width whose matrices have fragment-tiled copies: single tokens and short portions
+    (the tiled GEMM, K split into slabs for the narrow outputs) against whole prompts (library GEMMs)
+    and against the float32 restatement."""
+    eng = _engine("wide", dtype="bfloat16")
+    assert eng.runner._tiled_w, "no tiled weight copies at width 512"
+    toks = _tokens("wide", 48, 3)
+    want = _ref("wide", toks)
+    whole = _run_cuts(eng, "w", toks, [48])
+    for cuts in ([1] * 48, [20, 3, 1, 7] + [1] * 17):
+        got = _run_cuts(eng, "w", toks, cuts)
+        for a, b in ((got, want), (got, whole)):
+            d = a - b
+            d = d - d.mean(1, keepdims=True)
+            assert (np.sqrt((d ** 2).mean(1)) / np.abs(want).std()).max() < 0.08
+
+
+@pytest.mark.parametrize("name,dtype", [("loop0", "float32"), ("tail", "float32"), ("plain", "bfloat16"), ("wide", "bfloat16")])
 def test_greedy_generation_through_the_engine(name, dtype):
     """LLM.generate: scheduler admission, prefill, then decode steps replayed from HIP graphs with
     run-ahead.  A token may leave the restatement's only where its own margin is inside the error."""

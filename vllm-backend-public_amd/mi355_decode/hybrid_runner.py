@@ -167,6 +167,7 @@ class HybridRunner(ModelRunner):
         if self.Vp != self.V:
             self.head_w = torch.zeros(self.Vp, self.H, dtype=dtype, device=dev)
             self.head_w[: self.V] = weights.lm_head
+        self._init_tiled_copies(tiled_linears)
         self.logits_rows = torch.zeros(B, self.Vp, dtype=dtype, device=dev)
         self.logits = self.logits_rows[:, : self.V]
         self.graphs = {}
@@ -210,13 +211,42 @@ class HybridRunner(ModelRunner):
     def state_bytes_per_slot(self) -> int:
         return sum(t[0].numel() * t.element_size() for t in self.conv_state + self.rec_state)
 
+    def _init_tiled_copies(self, want: Optional[bool]) -> None:
+        """Fragment-tiled second copies of the wide matrices for the weight-streaming GEMM of decode-sized
+        steps (ModelRunner keeps the same kind of copy for its projections).  MI355_TILED_LINEARS=0 or
+        tiled_linears=False: none (the row-major stream, mi355_linear_decode, serves those steps)."""
+        import os
+        self._tiled_w = {}
+        if want is False or os.environ.get("MI355_TILED_LINEARS") == "0" or self.dtype == torch.float32:
+            return
+        mats = [self.head_w]
+        for lw in self.w.layers:
+            mats += [lw.in_w, lw.delta_o_w, lw.attn_o_w, lw.gate_up_w, lw.down_w, lw.a2_w, lw.g2_w]
+        for w in mats:
+            # the kernel stages x in 512-wide K slices; narrow outputs leave too few workgroups to pay
+            if w is not None and w.shape[1] % 512 == 0 and w.shape[0] >= 256 and w.shape[0] % 8 == 0:
+                self._tiled_w[w.data_ptr()] = ops.tile_weights(w)
+
     def linear(self, x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """x @ w.T: the weight-streaming kernel for decode-sized row counts where its layout rules
-        hold, a library GEMM otherwise (prefill; float32; odd widths)."""
+        """x @ w.T.  Decode-sized row counts stream the weights once: through the fragment-tiled copy
+        (K split over workgroups into fp32 slabs where one pass would leave most of the chip idle, a
+        second launch adds the slabs) or, for matrices that have none, row-major through
+        mi355_linear_decode.  A library GEMM otherwise (prefill; float32; odd widths)."""
         M, K = x.shape
         N = w.shape[0]
-        if (x.dtype != torch.float32 and M <= ops.LINEAR_DECODE_MAX_M and K % 32 == 0 and N % 4 == 0
-                and x.stride(1) == 1 and (M == 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0):
+        ok16 = x.dtype != torch.float32 and x.stride(1) == 1 and (M == 1 or x.stride(0) % 8 == 0) and x.data_ptr() % 16 == 0
+        tw = self._tiled_w.get(w.data_ptr()) if ok16 and M <= ops.LINEAR_DECODE_MAX_M else None
+        if tw is not None:
+            plan = ops.plan_linear_tiled(N, K, True, M)
+            if plan is not None:
+                tiles, groups = plan
+                if out is None:
+                    out = torch.empty(M, N, dtype=x.dtype, device=x.device)
+                if groups == 1:
+                    return ops.linear_tiled(x, tw, N, out=out, tiles_per_wg=tiles)
+                part = ops.linear_tiled(x, tw, N, tiles_per_wg=tiles, k_groups=groups, epilogue=ops.EPI_PARTIAL)
+                return ops.sum_slabs(part, groups, out)
+        if ok16 and M <= ops.LINEAR_DECODE_MAX_M and K % 32 == 0 and N % 4 == 0:
             return ops.linear_decode(x, w, None, out=out)
         if out is None:
             return torch.mm(x, w.t())
