@@ -746,7 +746,8 @@ int32_t mi355_allreduce_oneshot_destroy(void* comm);
  *   rms_norm_mix_f32      resid += alpha * (rmsnorm(xa) * wa + rmsnorm(xb) * wb); xb / wb may be null
  *   gelu_tanh_and_mul     out[t] = gelu_tanh(x[t, :inter]) * x[t, inter:2 inter]
  *   gated_head_rms_norm   out[t, h] = o[t, h] / rms(o[t, h]) * weight * act(gate[t, h]); o fp32
- *                         [tokens, heads, head_dim]; activation 0: silu, 1: sigmoid
+ *                         [tokens, heads, head_dim]; activation 0: silu, 1: sigmoid; weight [head_dim]
+ *                         shared by the heads (weight_heads 1) or [heads, head_dim] (weight_heads == heads)
  *   softcap               z = cap * tanh(z / cap), in place
  */
 int32_t mi355_embed_scale_f32(float* out, const void* embed, const int64_t* ids, int64_t num_tokens,
@@ -762,9 +763,9 @@ int32_t mi355_rms_norm_mix_f32(float* resid, const void* xa, const void* wa, con
 int32_t mi355_gelu_tanh_and_mul(void* out, const void* x, int64_t x_stride, int64_t num_tokens,
                                 int32_t inter, int32_t dtype, void* stream);
 int32_t mi355_gated_head_rms_norm(void* out, const float* o, const void* gate, int64_t gate_stride,
-                                  const float* weight, int64_t num_tokens, int32_t num_heads,
-                                  int32_t head_dim, float eps, int32_t activation, int32_t dtype,
-                                  void* stream);
+                                  const float* weight, int32_t weight_heads, int64_t num_tokens,
+                                  int32_t num_heads, int32_t head_dim, float eps, int32_t activation,
+                                  int32_t dtype, void* stream);
 int32_t mi355_softcap(void* z, int64_t numel, float cap, int32_t dtype, void* stream);
 
 /*
@@ -835,6 +836,113 @@ int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t stride, int32_
                                int32_t num_kv_heads, int32_t head_dim, int32_t v_dim,
                                int64_t num_tokens, float* workspace, int64_t workspace_floats,
                                int32_t dtype, void* stream);
+
+/*
+ * The general delta rule over the same packed chunks: state fp32 [slots, heads, head_dim, head_dim]
+ * (key channel, value channel; zero at position 0), per token and head
+ *     S <- diag(w) S - (a * u) (u^T S) + k v^T   (both first terms read the old S),   o = S^T r
+ *     w = exp(-exp(-1/2) * sigmoid(decay + decay_bias)),  a = sigmoid(rate + rate_bias),
+ *     u = k / sqrt(sum(k^2) + 1e-6)
+ * r / k / v / decay / rate are [tokens, heads * head_dim] activations (column slices are fine), the
+ * biases fp32 [heads * head_dim]; everything past the projections is fp32.  o is fp32
+ * [tokens, heads, head_dim].  workspace: mi355_general_delta_rule_workspace(...) floats.
+ */
+int64_t mi355_general_delta_rule_workspace(int64_t num_tokens, int32_t num_heads, int32_t head_dim);
+int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_stride, const void* k,
+                                 int64_t k_stride, const void* v, int64_t v_stride, const void* decay,
+                                 int64_t decay_stride, const float* decay_bias, const void* rate,
+                                 int64_t rate_stride, const float* rate_bias, float* state,
+                                 const int32_t* cu_seqlens, const int64_t* positions,
+                                 const int32_t* state_slots, int32_t num_seqs, int32_t num_heads,
+                                 int32_t head_dim, int64_t num_tokens, float* workspace,
+                                 int64_t workspace_floats, int32_t dtype, void* stream);
+
+/*
+ * More kernels on the fp32 residual stream.  gn(x): an RMS norm taken separately over each of
+ * `groups` equal consecutive parts of a row.
+ *   group_rms_norm_f32     gn(x) * weight for fp32 rows x, to activation rows `out` or to fp32 rows
+ *                          `out_f32` (exactly one of the two; out_f32 may be x)
+ *   gated_norm_resid_f32   resid += mult * gn(y * sigmoid(gate + bias)) * weight: y, gate activation
+ *                          rows (gate may be a column slice), bias / weight fp32 [width]
+ *   rms_norm_rows          out = x / sqrt(mean(x^2) + eps) * weight for rows of n columns (x may be a
+ *                          column slice), weight fp32 [n]
+ *   tanh_rows              out = tanh(x), the same shapes
+ */
+int32_t mi355_group_rms_norm_f32(void* out, float* out_f32, const float* x, const float* weight,
+                                 int64_t num_tokens, int32_t width, int32_t groups, float eps,
+                                 int32_t dtype, void* stream);
+int32_t mi355_gated_norm_resid_f32(float* resid, const void* y, const void* gate, int64_t gate_stride,
+                                   const float* bias, const float* weight, int64_t num_tokens,
+                                   int32_t width, int32_t groups, float eps, float mult, int32_t dtype,
+                                   void* stream);
+int32_t mi355_rms_norm_rows(void* out, const void* x, int64_t x_stride, const float* weight,
+                            int64_t num_rows, int32_t n, float eps, int32_t dtype, void* stream);
+int32_t mi355_tanh_rows(void* out, const void* x, int64_t x_stride, int64_t num_rows, int32_t n,
+                        int32_t dtype, void* stream);
+
+/*
+ * Attention through a low-rank latent.  Per token the pages hold the normed latent c [rank] and one
+ * rotated key part [rot] shared by all heads: cache [blocks, 16, rank + rot].
+ *   latent_kv_write      x [tokens, rank + rot] (a column slice is fine): c = x[:rank] / rms * norm_weight,
+ *                        the last rot columns rotated (first rot_dims of them, coordinate i with
+ *                        i + rot_dims / 2, table cos_sin [max_pos, rot_dims] = cos | sin), into the
+ *                        row's page slot; rows with slot < 0 store nothing
+ *   latent_window_attn   out[t, h] = sigmoid(gate[t, h]) * sum_j p_j c_j over the keys j of the row's
+ *                        sequence with 0 <= p - j < window,
+ *                        p_j = exp(s_j) / (exp(sink[h]) + sum_j' exp(s_j')),
+ *                        s_j = (q_latent[t, h] . c_j + rotate(q[t, h, q_rot_offset:]) . kr_j) * scale.
+ *                        q_latent is the query's unrotated part already multiplied into the latent
+ *                        space, rank numbers at q_latent + t * q_latent_stride + h * q_latent_head_stride
+ *                        (token-major or head-major); q [tokens, heads * q_head_width] holds the part to
+ *                        rotate at q_rot_offset of every head.  out: rank numbers per (t, h), strides
+ *                        likewise; the caller applies the value up-projection.  gate may be null.
+ */
+int32_t mi355_latent_kv_write(void* cache, const void* x, int64_t x_stride, const float* norm_weight,
+                              const float* cos_sin, int32_t max_pos, const int64_t* positions,
+                              const int64_t* slot_mapping, int64_t num_tokens, int32_t rank,
+                              int32_t rot, int32_t rot_dims, float eps, int32_t dtype, void* stream);
+int32_t mi355_latent_window_attn(void* out, int64_t out_stride, int64_t out_head_stride,
+                                 const void* q_latent, int64_t q_latent_stride,
+                                 int64_t q_latent_head_stride, const void* q, int64_t q_stride,
+                                 int32_t q_head_width,
+                                 int32_t q_rot_offset, const void* cache, const int32_t* block_tables,
+                                 int32_t max_blocks, const int32_t* tok_seq, const int64_t* positions,
+                                 const float* sink, const void* gate, int64_t gate_stride,
+                                 const float* cos_sin, int32_t max_pos, int64_t num_tokens,
+                                 int32_t num_heads, int32_t rank, int32_t rot, int32_t rot_dims,
+                                 int32_t window, float scale, int32_t dtype, void* stream);
+
+/*
+ * Mixture-of-experts feed-forward.  A routed row is (token t, choice k), number t * top + k.
+ *   moe_route         from fp32 router logits [tokens, experts]: score = sigmoid(logit); experts are
+ *                     chosen by score + correction among the experts of the `keep` best of `groups`
+ *                     groups of neighbouring experts (a group scores the sum of its two largest
+ *                     score + correction); ids [tokens, top], weights [tokens, top] = the chosen
+ *                     experts' scores (no correction, not renormalised)
+ *   moe_sort          routed rows by expert: offsets [experts + 1], perm[position] = row,
+ *                     inv[row] = position
+ *   moe_gather_rows   xs[position] = x[perm[position] / top]
+ *   moe_gate_up_rows  act[position] = silu(Wg[e] x[t]) * (Wu[e] x[t]); w_gate_up [experts, 2 ff, width]
+ *   moe_down_rows     y[position] = Wd[e] act[position]; w_down [experts, width, ff]
+ *   moe_silu_and_mul  out = silu(x[:, :ff]) * x[:, ff:]
+ *   moe_combine       out[t] = sum_k weights[t, k] * y[inv[t * top + k]]
+ */
+int32_t mi355_moe_route(int32_t* ids, float* weights, const float* logits, const float* correction,
+                        int64_t num_tokens, int32_t experts, int32_t top, int32_t groups, int32_t keep,
+                        void* stream);
+int32_t mi355_moe_sort(int32_t* offsets, int32_t* perm, int32_t* inv, const int32_t* ids,
+                       int64_t num_rows, int32_t experts, void* stream);
+int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t* perm, int64_t num_rows,
+                              int32_t top, int32_t width, int32_t dtype, void* stream);
+int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* w_gate_up, const int32_t* offsets,
+                               const int32_t* perm, int32_t experts, int32_t top, int32_t width,
+                               int32_t ff, int32_t dtype, void* stream);
+int32_t mi355_moe_down_rows(void* y, const void* act, const void* w_down, const int32_t* offsets,
+                            int32_t experts, int32_t width, int32_t ff, int32_t dtype, void* stream);
+int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_rows, int32_t ff, int32_t dtype,
+                               void* stream);
+int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights,
+                          int64_t num_tokens, int32_t top, int32_t width, int32_t dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,295 @@
+// Mixture-of-experts feed-forward: routing, the expert-sorted row order, and the expert products for
+// steps of few rows.
+//   moe_route           sigmoid scores from fp32 router logits; experts are picked by score + correction
+//                       among the experts of the best `keep` of `count` groups of neighbours (a group
+//                       scores the sum of its two best), and weighted by the score without correction
+//   moe_sort            rows (token, choice) ordered by expert: offsets[E + 1], perm[position] = row,
+//                       inv[row] = position
+//   moe_gather_rows     xs[position] = x[perm[position] / top]
+//   moe_gate_up_rows    a[position] = silu(Wg[e] x) * (Wu[e] x) for every routed row, one wave per
+//                       (expert, hidden unit) walking that expert's rows: an expert's weights leave HBM once
+//   moe_down_rows       y[position] = Wd[e] a[position], the same way
+//   moe_silu_and_mul    a = silu(gu[:, :F]) * gu[:, F:] (any storage type)
+//   moe_combine         out[t] = sum_k weight[t, k] * y[inv[t * top + k]]
+// Routing, scores and the weighted sum are fp32; activations and expert weights are stored in the
+// dtype argument's type, products accumulate in fp32.
+#include "common.h"
+
+namespace mi355 {
+
+constexpr int kMaxGroups = 64;
+constexpr int kMaxTop = 16;
+
+__global__ __launch_bounds__(64) void moe_route_kernel(int32_t* __restrict__ ids, float* __restrict__ wts,
+                                                       const float* __restrict__ z, const float* __restrict__ corr,
+                                                       int64_t T, int E, int top, int count, int keep) {
+  const int64_t t = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
+  if (t >= T) return;
+  const float* zr = z + t * E;
+  const int per = E / count;
+  const float ninf = -__builtin_inff();
+  auto choice = [&](int e) {
+    return 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + e))) + MI355_LD(float, corr, corr + e);
+  };
+  // the groups that stay: `keep` rounds of picking the best group not yet picked
+  uint64_t allowed = 0;
+  if (keep >= count) {
+    allowed = ~0ull;
+  } else {
+    for (int r = 0; r < keep; ++r) {
+      int best = -1;
+      float bs = ninf;
+      for (int g = 0; g < count; ++g) {
+        if ((allowed >> g) & 1ull) continue;
+        float a = ninf, b = ninf;                       // the two largest of the group
+        for (int i = 0; i < per; ++i) {
+          const float c = choice(g * per + i);
+          if (c > a) { b = a; a = c; } else if (c > b) { b = c; }
+        }
+        const float gs = per > 1 ? a + b : a;
+        if (best < 0 || gs > bs) { best = g; bs = gs; }
+      }
+      allowed |= 1ull << best;
+    }
+  }
+  int picked[kMaxTop];
+  for (int r = 0; r < top; ++r) {
+    int best = -1;
+    float bs = ninf;
+    for (int e = 0; e < E; ++e) {
+      if (!((allowed >> (e / per)) & 1ull)) continue;
+      bool taken = false;
+      for (int q = 0; q < r; ++q) taken |= picked[q] == e;
+      if (taken) continue;
+      const float c = choice(e);
+      if (best < 0 || c > bs) { best = e; bs = c; }
+    }
+    picked[r] = best;
+    MI355_ST(int32_t, ids, ids + t * top + r, best);
+    MI355_ST(float, wts, wts + t * top + r, 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + best))));
+  }
+}
+
+// one workgroup: counts, an exclusive prefix, then a position for every row
+__global__ __launch_bounds__(1024) void moe_sort_kernel(int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
+                                                        int32_t* __restrict__ inv, const int32_t* __restrict__ ids,
+                                                        int64_t rows, int E) {
+  extern __shared__ int32_t sm[];                       // counts [E] | starts [E + 1]
+  int32_t* cnt = sm;
+  int32_t* start = sm + E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) atomicAdd(&cnt[MI355_LD(int32_t, ids, ids + r)], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t at = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = at;
+      at += cnt[e];
+    }
+    start[E] = at;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e <= E; e += blockDim.x) MI355_ST(int32_t, offsets, offsets + e, start[e]);
+  __syncthreads();
+  // positions inside an expert's range are handed out in arrival order: which row lands where varies
+  // from run to run, what is computed for a row does not depend on it
+  for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) {
+    const int32_t at = atomicAdd(&start[MI355_LD(int32_t, ids, ids + r)], 1);
+    MI355_ST(int32_t, perm, perm + at, static_cast<int32_t>(r));
+    MI355_ST(int32_t, inv, inv + r, at);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gather_rows_kernel(typename Elem<T>::S* __restrict__ xs,
+                                                              const typename Elem<T>::S* __restrict__ x,
+                                                              const int32_t* __restrict__ perm, int top, int W) {
+  const int64_t p = blockIdx.x;
+  const int64_t t = MI355_LD(int32_t, perm, perm + p) / top;
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    MI355_ST(typename Elem<T>::S, xs, xs + p * W + c, MI355_LD(typename Elem<T>::S, x, x + t * W + c));
+}
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+// one wave per (expert, hidden unit f): gate and up rows of that unit against every row routed to the expert
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(typename Elem<T>::S* __restrict__ a,
+                                                               const typename Elem<T>::S* __restrict__ x,
+                                                               const typename Elem<T>::S* __restrict__ w_gate_up,
+                                                               const int32_t* __restrict__ offsets,
+                                                               const int32_t* __restrict__ perm, int top, int W, int F) {
+  const int e = blockIdx.y, lane = threadIdx.x & 63;
+  const int f = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (f >= F) return;
+  const int lo = MI355_LD(int32_t, offsets, offsets + e), hi = MI355_LD(int32_t, offsets, offsets + e + 1);
+  const typename Elem<T>::S* wg = w_gate_up + (static_cast<int64_t>(e) * 2 * F + f) * W;
+  const typename Elem<T>::S* wu = wg + static_cast<int64_t>(F) * W;
+  for (int p = lo; p < hi; ++p) {
+    const int64_t t = MI355_LD(int32_t, perm, perm + p) / top;
+    float g = 0.f, u = 0.f;
+    for (int c = lane; c < W; c += 64) {
+      const float xv = MI355_LDF(T, x, x + t * W + c);
+      g += xv * MI355_LDF(T, w_gate_up, wg + c);
+      u += xv * MI355_LDF(T, w_gate_up, wu + c);
+    }
+    g = wave_sum(g);
+    u = wave_sum(u);
+    if (lane == 0) {
+      const float gr = elem_to_f<T>(elem_from_f<T>(g)), ur = elem_to_f<T>(elem_from_f<T>(u));   // as stored by a product
+      MI355_STF(T, a, a + static_cast<int64_t>(p) * F + f, silu_f(gr) * ur);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_rows_kernel(typename Elem<T>::S* __restrict__ y,
+                                                            const typename Elem<T>::S* __restrict__ a,
+                                                            const typename Elem<T>::S* __restrict__ w_down,
+                                                            const int32_t* __restrict__ offsets, int W, int F) {
+  const int e = blockIdx.y, lane = threadIdx.x & 63;
+  const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (c >= W) return;
+  const int lo = MI355_LD(int32_t, offsets, offsets + e), hi = MI355_LD(int32_t, offsets, offsets + e + 1);
+  const typename Elem<T>::S* wd = w_down + (static_cast<int64_t>(e) * W + c) * F;
+  for (int p = lo; p < hi; ++p) {
+    float s = 0.f;
+    for (int f = lane; f < F; f += 64)
+      s += MI355_LDF(T, a, a + static_cast<int64_t>(p) * F + f) * MI355_LDF(T, w_down, wd + f);
+    s = wave_sum(s);
+    if (lane == 0) MI355_STF(T, y, y + static_cast<int64_t>(p) * W + c, s);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_silu_and_mul_kernel(typename Elem<T>::S* __restrict__ out,
+                                                               const typename Elem<T>::S* __restrict__ x, int64_t rows,
+                                                               int F) {
+  const int64_t total = rows * F;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t r = i / F;
+    const int f = static_cast<int>(i % F);
+    MI355_STF(T, out, out + i, silu_f(MI355_LDF(T, x, x + r * 2 * F + f)) * MI355_LDF(T, x, x + r * 2 * F + F + f));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(typename Elem<T>::S* __restrict__ out,
+                                                          const typename Elem<T>::S* __restrict__ y,
+                                                          const int32_t* __restrict__ inv, const float* __restrict__ wts,
+                                                          int top, int W) {
+  const int64_t t = blockIdx.x;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float s = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int64_t p = MI355_LD(int32_t, inv, inv + t * top + k);
+      s += MI355_LD(float, wts, wts + t * top + k) * MI355_LDF(T, y, y + p * W + c);
+    }
+    MI355_STF(T, out, out + t * W + c, s);
+  }
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+#define REQ_DTYPE(dtype) MI355_REQUIRE((dtype) >= MI355_BF16 && (dtype) <= MI355_F32, MI355_ERR_UNSUPPORTED, "dtype code %d", (dtype))
+
+extern "C" int32_t mi355_moe_route(int32_t* ids, float* weights, const float* logits, const float* correction,
+                                   int64_t num_tokens, int32_t experts, int32_t top, int32_t groups, int32_t keep,
+                                   void* stream) {
+  MI355_REQUIRE(ids && weights && logits && correction, MI355_ERR_INVALID, "moe_route: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && experts > 0 && top > 0 && groups > 0 && keep > 0 && keep <= groups &&
+                    experts % groups == 0,
+                MI355_ERR_INVALID, "moe_route: %d experts in %d groups, %d kept, %d chosen", experts, groups, keep, top);
+  MI355_REQUIRE(top <= kMaxTop && groups <= kMaxGroups && top <= keep * (experts / groups), MI355_ERR_UNSUPPORTED,
+                "moe_route: at most %d chosen experts and %d groups; the kept groups must hold the %d chosen", kMaxTop,
+                kMaxGroups, top);
+  if (num_tokens == 0) return MI355_OK;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((num_tokens + 63) / 64)), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), ids, weights, logits, correction, num_tokens, experts, top, groups,
+                     keep);
+  return check_launch("moe_route");
+}
+
+extern "C" int32_t mi355_moe_sort(int32_t* offsets, int32_t* perm, int32_t* inv, const int32_t* ids, int64_t num_rows,
+                                  int32_t experts, void* stream) {
+  MI355_REQUIRE(offsets && perm && inv && ids, MI355_ERR_INVALID, "moe_sort: null pointer");
+  MI355_REQUIRE(num_rows >= 0 && num_rows <= 0x7FFFFFFF && experts > 0 && experts <= 4096, MI355_ERR_INVALID,
+                "moe_sort: sizes");
+  hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), (2 * static_cast<size_t>(experts) + 1) * sizeof(int32_t),
+                     static_cast<hipStream_t>(stream), offsets, perm, inv, ids, num_rows, experts);
+  return check_launch("moe_sort");
+}
+
+extern "C" int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t* perm, int64_t num_rows, int32_t top,
+                                         int32_t width, int32_t dtype, void* stream) {
+  MI355_REQUIRE(xs && x && perm, MI355_ERR_INVALID, "moe_gather_rows: null pointer");
+  MI355_REQUIRE(num_rows >= 0 && top > 0 && width > 0, MI355_ERR_INVALID, "moe_gather_rows: sizes");
+  REQ_DTYPE(dtype);
+  if (num_rows == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_gather_rows_kernel<TT>), dim3(num_rows), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(xs), static_cast<const Elem<TT>::S*>(x), perm,
+                                                  top, width));
+  return check_launch("moe_gather_rows");
+}
+
+extern "C" int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* w_gate_up, const int32_t* offsets,
+                                          const int32_t* perm, int32_t experts, int32_t top, int32_t width, int32_t ff,
+                                          int32_t dtype, void* stream) {
+  MI355_REQUIRE(act && x && w_gate_up && offsets && perm, MI355_ERR_INVALID, "moe_gate_up_rows: null pointer");
+  MI355_REQUIRE(experts > 0 && experts <= 65535 && top > 0 && width > 0 && ff > 0, MI355_ERR_INVALID,
+                "moe_gate_up_rows: sizes");
+  REQ_DTYPE(dtype);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>((ff + 3) / 4), static_cast<unsigned>(experts));
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_gate_up_rows_kernel<TT>), grid, dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(act), static_cast<const Elem<TT>::S*>(x),
+                                                  static_cast<const Elem<TT>::S*>(w_gate_up), offsets, perm, top, width,
+                                                  ff));
+  return check_launch("moe_gate_up_rows");
+}
+
+extern "C" int32_t mi355_moe_down_rows(void* y, const void* act, const void* w_down, const int32_t* offsets,
+                                       int32_t experts, int32_t width, int32_t ff, int32_t dtype, void* stream) {
+  MI355_REQUIRE(y && act && w_down && offsets, MI355_ERR_INVALID, "moe_down_rows: null pointer");
+  MI355_REQUIRE(experts > 0 && experts <= 65535 && width > 0 && ff > 0, MI355_ERR_INVALID, "moe_down_rows: sizes");
+  REQ_DTYPE(dtype);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>((width + 3) / 4), static_cast<unsigned>(experts));
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_down_rows_kernel<TT>), grid, dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(y), static_cast<const Elem<TT>::S*>(act),
+                                                  static_cast<const Elem<TT>::S*>(w_down), offsets, width, ff));
+  return check_launch("moe_down_rows");
+}
+
+extern "C" int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_rows, int32_t ff, int32_t dtype,
+                                          void* stream) {
+  MI355_REQUIRE(out && x, MI355_ERR_INVALID, "moe_silu_and_mul: null pointer");
+  MI355_REQUIRE(num_rows >= 0 && ff > 0, MI355_ERR_INVALID, "moe_silu_and_mul: sizes");
+  REQ_DTYPE(dtype);
+  if (num_rows == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t blocks = (num_rows * ff + 255) / 256;
+  const dim3 grid(static_cast<unsigned>(blocks > 65536 ? 65536 : blocks));
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_silu_and_mul_kernel<TT>), grid, dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(x),
+                                                  num_rows, ff));
+  return check_launch("moe_silu_and_mul");
+}
+
+extern "C" int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights,
+                                     int64_t num_tokens, int32_t top, int32_t width, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && y && inv && weights, MI355_ERR_INVALID, "moe_combine: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && top > 0 && width > 0, MI355_ERR_INVALID, "moe_combine: sizes");
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_combine_kernel<TT>), dim3(num_tokens), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(y), inv,
+                                                  weights, top, width));
+  return check_launch("moe_combine");
+}

@@ -6,6 +6,12 @@
 //   gelu_tanh_and_mul        out = gelu_tanh(gate) * up for rows holding gate | up
 //   gated_head_rms_norm      out = o / rms(o) * w * act(gate) per (token, head) row of an fp32 tensor
 //   softcap                  z = cap * tanh(z / cap)
+//   group_rms_norm_f32       out = gn(x) * w: an RMS norm over each of `groups` equal consecutive parts of an
+//                            fp32 row, to activation rows or (in place or not) to fp32 rows
+//   gated_norm_resid_f32     resid += mult * gn(y * sigmoid(g + b)) * w: a sub-layer's result, gated element by
+//                            element, normed in groups, scaled, added to the fp32 residual
+//   rms_norm_rows            out = x / rms(x) * w for short rows that may be column slices (fp32 weight)
+//   tanh_rows                out = tanh(x) for rows that may be column slices
 // Every sum, mean and transcendental is fp32; activations are stored in bf16, fp16 or fp32
 // (the dtype argument).  HBM-bound: one pass over the rows, one workgroup (or one wave) per row.
 #include "common.h"
@@ -140,7 +146,8 @@ __global__ __launch_bounds__(256) void gated_head_rms_norm_kernel(typename Elem<
                                                                   const float* __restrict__ o,
                                                                   const typename Elem<T>::S* __restrict__ gate,
                                                                   int64_t gate_stride, const float* __restrict__ w,
-                                                                  int64_t rows, int H, int dv, float eps, int act) {
+                                                                  int w_heads, int64_t rows, int H, int dv, float eps,
+                                                                  int act) {
   const int64_t row = blockIdx.x * static_cast<int64_t>(blockDim.x >> 6) + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int lane = threadIdx.x & 63;
@@ -158,7 +165,7 @@ __global__ __launch_bounds__(256) void gated_head_rms_norm_kernel(typename Elem<
     const float g = MI355_LDF(T, gate, gate + t * gate_stride + static_cast<int64_t>(h) * dv + c);
     const float s = 1.0f / (1.0f + expf(-g));
     const float a = act == 0 ? g * s : s;
-    MI355_STF(T, out, out + row * dv + c, v * r * MI355_LD(float, w, w + c) * a);
+    MI355_STF(T, out, out + row * dv + c, v * r * MI355_LD(float, w, w + (w_heads > 1 ? h * dv : 0) + c) * a);
   }
 }
 
@@ -167,6 +174,88 @@ __global__ __launch_bounds__(256) void softcap_kernel(typename Elem<T>::S* __res
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x)
     MI355_STF(T, z, z + i, cap * tanhf(MI355_LDF(T, z, z + i) / cap));
+}
+
+constexpr int kMaxNormGroups = 64;
+
+// rg[g] = 1 / sqrt(mean of sq(c) over the columns c of group g + eps), for every group of gw columns
+template <typename F>
+__device__ __forceinline__ void group_rsqrt(F sq, int groups, int gw, float eps, float* rg, float* scratch) {
+  for (int g = 0; g < groups; ++g) {
+    float s = 0.f;
+    for (int c = g * gw + threadIdx.x; c < (g + 1) * gw; c += blockDim.x) s += sq(c);
+    s = block_sum32(s, scratch);
+    if (threadIdx.x == 0) rg[g] = 1.0f / sqrtf(s / static_cast<float>(gw) + eps);
+  }
+  __syncthreads();
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void group_rms_norm_f32_kernel(typename Elem<T>::S* __restrict__ out,
+                                                                 float* out_f32, const float* x,   // may be one buffer
+                                                                 const float* __restrict__ weight, int W, int groups,
+                                                                 float eps) {
+  __shared__ float scratch[32];
+  __shared__ float rg[kMaxNormGroups];
+  const int64_t t = blockIdx.x;
+  const int gw = W / groups;
+  group_rsqrt([&](int c) { const float v = MI355_LD(float, x, x + t * W + c); return v * v; }, groups, gw, eps, rg, scratch);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = MI355_LD(float, x, x + t * W + c) * rg[c / gw] * MI355_LD(float, weight, weight + c);
+    if (out_f32 != nullptr) MI355_ST(float, out_f32, out_f32 + t * W + c, v);
+    else MI355_STF(T, out, out + t * W + c, v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gated_norm_resid_f32_kernel(float* __restrict__ resid,
+                                                                   const typename Elem<T>::S* __restrict__ y,
+                                                                   const typename Elem<T>::S* __restrict__ gate,
+                                                                   int64_t gate_stride, const float* __restrict__ bias,
+                                                                   const float* __restrict__ weight, int W, int groups,
+                                                                   float eps, float mult) {
+  __shared__ float scratch[32];
+  __shared__ float rg[kMaxNormGroups];
+  const int64_t t = blockIdx.x;
+  const int gw = W / groups;
+  auto gated = [&](int c) {
+    const float z = MI355_LDF(T, gate, gate + t * gate_stride + c) + MI355_LD(float, bias, bias + c);
+    return MI355_LDF(T, y, y + t * W + c) / (1.0f + expf(-z));
+  };
+  group_rsqrt([&](int c) { const float v = gated(c); return v * v; }, groups, gw, eps, rg, scratch);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = gated(c) * rg[c / gw] * MI355_LD(float, weight, weight + c);
+    MI355_ST(float, resid, resid + t * W + c, MI355_LD(float, resid, resid + t * W + c) + mult * v);
+  }
+}
+
+// one wave per row
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_rows_kernel(typename Elem<T>::S* __restrict__ out,
+                                                            const typename Elem<T>::S* __restrict__ x, int64_t x_stride,
+                                                            const float* __restrict__ weight, int64_t rows, int n,
+                                                            float eps) {
+  const int64_t row = blockIdx.x * static_cast<int64_t>(blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  float ss = 0.f;
+  for (int c = lane; c < n; c += 64) {
+    const float v = MI355_LDF(T, x, x + row * x_stride + c);
+    ss += v * v;
+  }
+  const float r = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(n) + eps);
+  for (int c = lane; c < n; c += 64)
+    MI355_STF(T, out, out + row * n + c, MI355_LDF(T, x, x + row * x_stride + c) * r * MI355_LD(float, weight, weight + c));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void tanh_rows_kernel(typename Elem<T>::S* __restrict__ out,
+                                                        const typename Elem<T>::S* __restrict__ x, int64_t x_stride,
+                                                        int64_t rows, int n) {
+  const int64_t total = rows * n;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    MI355_STF(T, out, out + i, tanhf(MI355_LDF(T, x, x + (i / n) * x_stride + i % n)));
 }
 
 static inline dim3 stride_grid(int64_t total) {
@@ -263,23 +352,25 @@ extern "C" int32_t mi355_gelu_tanh_and_mul(void* out, const void* x, int64_t x_s
 }
 
 extern "C" int32_t mi355_gated_head_rms_norm(void* out, const float* o, const void* gate, int64_t gate_stride,
-                                             const float* weight, int64_t num_tokens, int32_t num_heads,
-                                             int32_t head_dim, float eps, int32_t activation, int32_t dtype,
-                                             void* stream) {
+                                             const float* weight, int32_t weight_heads, int64_t num_tokens,
+                                             int32_t num_heads, int32_t head_dim, float eps, int32_t activation,
+                                             int32_t dtype, void* stream) {
   MI355_REQUIRE(out && o && gate && weight, MI355_ERR_INVALID, "gated_head_rms_norm: null pointer");
   MI355_REQUIRE(num_tokens >= 0 && num_heads > 0 && head_dim > 0 &&
                     gate_stride >= static_cast<int64_t>(num_heads) * head_dim,
                 MI355_ERR_INVALID, "gated_head_rms_norm: sizes");
   MI355_REQUIRE(activation == 0 || activation == 1, MI355_ERR_INVALID,
                 "gated_head_rms_norm: activation is 0 (silu) or 1 (sigmoid)");
+  MI355_REQUIRE(weight_heads == 1 || weight_heads == num_heads, MI355_ERR_INVALID,
+                "gated_head_rms_norm: the weight is one head's (1) or all heads' (%d), not %d", num_heads, weight_heads);
   REQ_DTYPE(dtype);
   const int64_t rows = num_tokens * num_heads;
   if (rows == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((gated_head_rms_norm_kernel<TT>), dim3((rows + 3) / 4), dim3(256), 0, s,
                                                   static_cast<Elem<TT>::S*>(out), o,
-                                                  static_cast<const Elem<TT>::S*>(gate), gate_stride, weight, rows,
-                                                  num_heads, head_dim, eps, activation));
+                                                  static_cast<const Elem<TT>::S*>(gate), gate_stride, weight,
+                                                  weight_heads, rows, num_heads, head_dim, eps, activation));
   return check_launch("gated_head_rms_norm");
 }
 
@@ -292,4 +383,63 @@ extern "C" int32_t mi355_softcap(void* z, int64_t numel, float cap, int32_t dtyp
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((softcap_kernel<TT>), stride_grid(numel), dim3(256), 0, s,
                                                   static_cast<Elem<TT>::S*>(z), numel, cap));
   return check_launch("softcap");
+}
+
+extern "C" int32_t mi355_group_rms_norm_f32(void* out, float* out_f32, const float* x, const float* weight,
+                                            int64_t num_tokens, int32_t width, int32_t groups, float eps, int32_t dtype,
+                                            void* stream) {
+  MI355_REQUIRE((out != nullptr) != (out_f32 != nullptr) && x && weight, MI355_ERR_INVALID,
+                "group_rms_norm_f32: null pointer, or both outputs given");
+  MI355_REQUIRE(num_tokens >= 0 && width > 0 && groups > 0 && groups <= kMaxNormGroups && width % groups == 0,
+                MI355_ERR_INVALID, "group_rms_norm_f32: width %d in %d groups (at most %d)", width, groups, kMaxNormGroups);
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((group_rms_norm_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), out_f32, x, weight, width, groups, eps));
+  return check_launch("group_rms_norm_f32");
+}
+
+extern "C" int32_t mi355_gated_norm_resid_f32(float* resid, const void* y, const void* gate, int64_t gate_stride,
+                                              const float* bias, const float* weight, int64_t num_tokens, int32_t width,
+                                              int32_t groups, float eps, float mult, int32_t dtype, void* stream) {
+  MI355_REQUIRE(resid && y && gate && bias && weight, MI355_ERR_INVALID, "gated_norm_resid_f32: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && width > 0 && groups > 0 && groups <= kMaxNormGroups && width % groups == 0 &&
+                    gate_stride >= width,
+                MI355_ERR_INVALID, "gated_norm_resid_f32: width %d in %d groups (at most %d)", width, groups,
+                kMaxNormGroups);
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((gated_norm_resid_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s,
+                                                  resid, static_cast<const Elem<TT>::S*>(y),
+                                                  static_cast<const Elem<TT>::S*>(gate), gate_stride, bias, weight, width,
+                                                  groups, eps, mult));
+  return check_launch("gated_norm_resid_f32");
+}
+
+extern "C" int32_t mi355_rms_norm_rows(void* out, const void* x, int64_t x_stride, const float* weight, int64_t num_rows,
+                                       int32_t n, float eps, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && x && weight, MI355_ERR_INVALID, "rms_norm_rows: null pointer");
+  MI355_REQUIRE(num_rows >= 0 && n > 0 && x_stride >= n, MI355_ERR_INVALID, "rms_norm_rows: sizes");
+  REQ_DTYPE(dtype);
+  if (num_rows == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((rms_norm_rows_kernel<TT>), dim3((num_rows + 3) / 4), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(x),
+                                                  x_stride, weight, num_rows, n, eps));
+  return check_launch("rms_norm_rows");
+}
+
+extern "C" int32_t mi355_tanh_rows(void* out, const void* x, int64_t x_stride, int64_t num_rows, int32_t n, int32_t dtype,
+                                   void* stream) {
+  MI355_REQUIRE(out && x, MI355_ERR_INVALID, "tanh_rows: null pointer");
+  MI355_REQUIRE(num_rows >= 0 && n > 0 && x_stride >= n, MI355_ERR_INVALID, "tanh_rows: sizes");
+  REQ_DTYPE(dtype);
+  if (num_rows == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((tanh_rows_kernel<TT>), stride_grid(num_rows * n), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(x),
+                                                  x_stride, num_rows, n));
+  return check_launch("tanh_rows");
 }

@@ -15,6 +15,7 @@
 //   causal_conv_silu        y[t,c] = silu(sum_j w[c,j] x[t - (taps-1-j), c]), inputs before the chunk from the state
 //   conv_state_update       state <- the last taps-1 inputs of each sequence
 //   gated_delta_rule        S <- a S; u = b (v - S^T k); S <- S + k u^T; o = S^T q   per token and head
+//   general_delta_rule      S <- diag(w) S - (a * u) (u^T S) + k v^T; o = S^T r      per token and head
 #include "common.h"
 
 namespace mi355 {
@@ -613,6 +614,136 @@ __global__ __launch_bounds__(64) void gated_delta_rule_split_kernel(
   }
 }
 
+// ---- the general delta rule ------------------------------------------------------------------------
+// State S [d, d] per head (key channel i, value channel j), a decay per key channel and a removal
+// along the unit key, both terms on the OLD state:
+//     S <- diag(w) S - (a * u) (u^T S) + k v^T,   o = S^T r
+//     w = exp(-e^(-1/2) sigmoid(wl + w0)),  a = sigmoid(al + ab),  u = k / sqrt(|k|^2 + 1e-6)
+// wl / al are projection outputs; everything after them is fp32.  general_delta_prep_kernel computes
+// w, u, a * u (and fp32 copies of k and r) for every token and head into rows padded to dp; the
+// recurrence kernel splits the d rows of a state column over R adjacent lanes as above.
+template <typename T>
+__global__ __launch_bounds__(64) void general_delta_prep_kernel(
+    float* __restrict__ ws, const typename Elem<T>::S* __restrict__ r, int64_t r_stride,
+    const typename Elem<T>::S* __restrict__ k, int64_t k_stride, const typename Elem<T>::S* __restrict__ wl,
+    int64_t wl_stride, const float* __restrict__ w0, const typename Elem<T>::S* __restrict__ al, int64_t al_stride,
+    const float* __restrict__ ab, int H, int d, int dp) {
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const typename Elem<T>::S* kr = k + t * k_stride + static_cast<int64_t>(h) * d;
+  float kk = 0.f;
+  for (int c = lane; c < d; c += 64) {
+    const float kv = MI355_LDF(T, k, kr + c);
+    kk += kv * kv;
+  }
+  kk = 1.0f / sqrtf(wave_sum(kk) + 1e-6f);
+  float* o = ws + (t * H + h) * 5 * dp;                  // w | u | a u | k | r
+  for (int c = lane; c < dp; c += 64) {
+    float w = 1.f, u = 0.f, au = 0.f, kv = 0.f, rv = 0.f;
+    if (c < d) {
+      const int64_t hc = static_cast<int64_t>(h) * d + c;
+      kv = MI355_LDF(T, k, kr + c);
+      rv = MI355_LDF(T, r, r + t * r_stride + hc);
+      u = kv * kk;
+      const float zw = MI355_LDF(T, wl, wl + t * wl_stride + hc) + MI355_LD(float, w0, w0 + hc);
+      w = expf(-0.6065306597126334f / (1.0f + expf(-zw)));
+      const float za = MI355_LDF(T, al, al + t * al_stride + hc) + MI355_LD(float, ab, ab + hc);
+      au = u / (1.0f + expf(-za));
+    }
+    MI355_ST(float, ws, o + c, w);
+    MI355_ST(float, ws, o + dp + c, u);
+    MI355_ST(float, ws, o + 2 * dp + c, au);
+    MI355_ST(float, ws, o + 3 * dp + c, kv);
+    MI355_ST(float, ws, o + 4 * dp + c, rv);
+  }
+}
+
+template <typename T, int R, int DR, int PF>
+__global__ __launch_bounds__(64) void general_delta_rule_kernel(
+    float* __restrict__ o, const typename Elem<T>::S* __restrict__ v, int64_t v_stride, const float* __restrict__ ws,
+    float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int64_t* __restrict__ positions,
+    const int32_t* __restrict__ state_slots, int H, int d) {
+  constexpr int dp = R * DR;
+  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int r = lane & (R - 1), col = blockIdx.z * (64 / R) + lane / R;
+  const int64_t cs = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s);
+  const int64_t n = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1) - cs;
+  if (n <= 0) return;
+  const int64_t slot = MI355_LD(int32_t, state_slots, state_slots + s);
+  float* sp = state + ((slot * H + h) * d) * d;
+  const bool live = col < d;
+  const bool fresh = MI355_LD(int64_t, positions, positions + cs) == 0;
+  float S[DR];
+#pragma unroll
+  for (int j = 0; j < DR; ++j) {
+    const int i = r * DR + j;
+    S[j] = (live && !fresh && i < d) ? MI355_LD(float, state, sp + static_cast<int64_t>(i) * d + col) : 0.f;
+  }
+  struct Rows {
+    float w[PF][DR], u[PF][DR], au[PF][DR], k[PF][DR], r[PF][DR], v[PF];
+  };
+  Rows A, B;
+  auto fetch = [&](Rows& x, int64_t first) {
+#pragma unroll
+    for (int q = 0; q < PF; ++q) {
+      int64_t t = first + q;
+      if (t > cs + n - 1) t = cs + n - 1;               // past the chunk: a row that is loaded and not used
+      const float* p = ws + (t * H + h) * 5 * dp + r * DR;
+#pragma unroll
+      for (int j = 0; j < DR; j += 4) {
+        const float4 a4 = MI355_LD(float4, ws, p + j), b4 = MI355_LD(float4, ws, p + dp + j),
+                     c4 = MI355_LD(float4, ws, p + 2 * dp + j), d4 = MI355_LD(float4, ws, p + 3 * dp + j),
+                     e4 = MI355_LD(float4, ws, p + 4 * dp + j);
+        x.w[q][j] = a4.x, x.w[q][j + 1] = a4.y, x.w[q][j + 2] = a4.z, x.w[q][j + 3] = a4.w;
+        x.u[q][j] = b4.x, x.u[q][j + 1] = b4.y, x.u[q][j + 2] = b4.z, x.u[q][j + 3] = b4.w;
+        x.au[q][j] = c4.x, x.au[q][j + 1] = c4.y, x.au[q][j + 2] = c4.z, x.au[q][j + 3] = c4.w;
+        x.k[q][j] = d4.x, x.k[q][j + 1] = d4.y, x.k[q][j + 2] = d4.z, x.k[q][j + 3] = d4.w;
+        x.r[q][j] = e4.x, x.r[q][j + 1] = e4.y, x.r[q][j + 2] = e4.z, x.r[q][j + 3] = e4.w;
+      }
+      x.v[q] = live ? MI355_LDF(T, v, v + t * v_stride + static_cast<int64_t>(h) * d + col) : 0.f;
+    }
+  };
+  auto work = [&](const Rows& x, int64_t i0) {
+#pragma unroll
+    for (int q = 0; q < PF; ++q) {
+      if (i0 + q >= n) break;
+      float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+      for (int j = 0; j < DR; j += 2) {
+        d0 += S[j] * x.u[q][j];
+        d1 += S[j + 1] * x.u[q][j + 1];
+      }
+      const float dot = sum_lanes<R>(d0 + d1);          // u^T S of this column, from the old state
+      const float vj = x.v[q];
+      float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int j = 0; j < DR; j += 2) {
+        S[j] = x.w[q][j] * S[j] - x.au[q][j] * dot + x.k[q][j] * vj;
+        S[j + 1] = x.w[q][j + 1] * S[j + 1] - x.au[q][j + 1] * dot + x.k[q][j + 1] * vj;
+        o0 += S[j] * x.r[q][j];
+        o1 += S[j + 1] * x.r[q][j + 1];
+      }
+      const float out = sum_lanes<R>(o0 + o1);
+      if (live && r == 0) MI355_ST(float, o, o + ((cs + i0 + q) * H + h) * d + col, out);
+    }
+  };
+  fetch(A, cs);
+  for (int64_t i0 = 0; i0 < n; i0 += 2 * PF) {
+    if (i0 + PF < n) fetch(B, cs + i0 + PF);
+    work(A, i0);
+    if (i0 + PF >= n) break;
+    if (i0 + 2 * PF < n) fetch(A, cs + i0 + 2 * PF);
+    work(B, i0 + PF);
+  }
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < DR; ++j) {
+      const int i = r * DR + j;
+      if (i < d) MI355_ST(float, state, sp + static_cast<int64_t>(i) * d + col, S[j]);
+    }
+  }
+}
+
 // out = sigmoid(gate) * sum of the key-range partial sums of sigmoid_window_attn_mfma_kernel
 template <typename T>
 __global__ __launch_bounds__(256) void window_attn_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial,
@@ -879,4 +1010,59 @@ extern "C" int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t str
                                                decay_stride, a_log, dt_bias, per_channel, state, cu_seqlens, positions,
                                                state_slots, num_seqs, num_heads, num_kv_heads, head_dim, v_dim));
   return check_launch("gated_delta_rule");
+}
+
+static inline int64_t general_delta_dp(int head_dim) { return head_dim <= 32 ? 32 : head_dim <= 64 ? 64 : head_dim <= 128 ? 128 : 256; }
+
+extern "C" int64_t mi355_general_delta_rule_workspace(int64_t num_tokens, int32_t num_heads, int32_t head_dim) {
+  return num_tokens * num_heads * 5 * general_delta_dp(head_dim);
+}
+
+extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_stride, const void* k, int64_t k_stride,
+                                            const void* v, int64_t v_stride, const void* decay, int64_t decay_stride,
+                                            const float* decay_bias, const void* rate, int64_t rate_stride,
+                                            const float* rate_bias, float* state, const int32_t* cu_seqlens,
+                                            const int64_t* positions, const int32_t* state_slots, int32_t num_seqs,
+                                            int32_t num_heads, int32_t head_dim, int64_t num_tokens, float* workspace,
+                                            int64_t workspace_floats, int32_t dtype, void* stream) {
+  MI355_REQUIRE(o && r && k && v && decay && decay_bias && rate && rate_bias && state && cu_seqlens && positions &&
+                    state_slots && workspace,
+                MI355_ERR_INVALID, "general_delta_rule: null pointer");
+  MI355_REQUIRE(num_seqs >= 0 && num_tokens >= 0 && num_heads > 0 && head_dim > 0, MI355_ERR_INVALID,
+                "general_delta_rule: sizes");
+  MI355_REQUIRE(head_dim <= 256 && num_heads <= 65535, MI355_ERR_UNSUPPORTED,
+                "general_delta_rule: head_dim %d (at most 256)", head_dim);
+  const int64_t width = static_cast<int64_t>(num_heads) * head_dim;
+  MI355_REQUIRE(r_stride >= width && k_stride >= width && v_stride >= width && decay_stride >= width && rate_stride >= width,
+                MI355_ERR_INVALID, "general_delta_rule: row strides shorter than the rows");
+  REQ_DTYPE(dtype);
+  if (num_seqs == 0 || num_tokens == 0) return MI355_OK;
+  const int64_t dp = general_delta_dp(head_dim);
+  const int64_t need = mi355_general_delta_rule_workspace(num_tokens, num_heads, head_dim);
+  MI355_REQUIRE(workspace_floats >= need && aligned16(workspace), MI355_ERR_INVALID,
+                "general_delta_rule: workspace of %lld floats, %lld needed, 16-byte aligned",
+                static_cast<long long>(workspace_floats), static_cast<long long>(need));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int lanes = head_dim <= 32 ? 8 : 16;
+  const int cols = 64 / lanes;
+  const dim3 pgrid(static_cast<unsigned>(num_tokens), static_cast<unsigned>(num_heads));
+  const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads),
+                  static_cast<unsigned>((head_dim + cols - 1) / cols));
+#define MI355_GDELTA(TT, R, DR, PF)                                                                                  \
+  hipLaunchKernelGGL((general_delta_rule_kernel<TT, R, DR, PF>), grid, dim3(64), 0, s, o,                            \
+                     static_cast<const Elem<TT>::S*>(v), v_stride, workspace, state, cu_seqlens, positions,          \
+                     state_slots, num_heads, head_dim)
+  MI355_DISPATCH_DTYPE3(dtype, {
+    typedef Elem<TT>::S E;
+    hipLaunchKernelGGL((general_delta_prep_kernel<TT>), pgrid, dim3(64), 0, s, workspace, static_cast<const E*>(r),
+                       r_stride, static_cast<const E*>(k), k_stride, static_cast<const E*>(decay), decay_stride,
+                       decay_bias, static_cast<const E*>(rate), rate_stride, rate_bias, num_heads, head_dim,
+                       static_cast<int>(dp));
+    if (dp == 32) MI355_GDELTA(TT, 8, 4, 4);
+    else if (dp == 64) MI355_GDELTA(TT, 16, 4, 4);
+    else if (dp == 128) MI355_GDELTA(TT, 16, 8, 2);
+    else MI355_GDELTA(TT, 16, 16, 1);
+  });
+#undef MI355_GDELTA
+  return check_launch("general_delta_rule");
 }

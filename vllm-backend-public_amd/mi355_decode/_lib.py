@@ -101,7 +101,7 @@ def _load() -> ctypes.CDLL:
         "mi355_add_rms_norm_f32": (I32, [P, P, P, P, I32, I64, I32, F, I32, P]),
         "mi355_rms_norm_mix_f32": (I32, [P, P, P, P, P, I64, I32, F, F, I32, P]),
         "mi355_gelu_tanh_and_mul": (I32, [P, P, I64, I64, I32, I32, P]),
-        "mi355_gated_head_rms_norm": (I32, [P, P, P, I64, P, I64, I32, I32, F, I32, I32, P]),
+        "mi355_gated_head_rms_norm": (I32, [P, P, P, I64, P, I32, I64, I32, I32, F, I32, I32, P]),
         "mi355_softcap": (I32, [P, I64, F, I32, P]),
         "mi355_rope_partial_kv_write": (I32, [P, I64, P, I64, P, I64, P, I32, P, P, P, P, I64, I32, I32, I32, I32, I32,
                                               I32, P]),
@@ -112,6 +112,23 @@ def _load() -> ctypes.CDLL:
         "mi355_gated_delta_rule": (I32, [P, P, I64, I32, I32, I32, P, I64, P, I64, P, P, I32, P, P, P, P, I32, I32, I32,
                                          I32, I32, I64, P, I64, I32, P]),
         "mi355_gated_delta_rule_workspace": (I64, [I64, I32, I32, I32]),
+        "mi355_general_delta_rule_workspace": (I64, [I64, I32, I32]),
+        "mi355_general_delta_rule": (I32, [P, P, I64, P, I64, P, I64, P, I64, P, P, I64, P, P, P, P, P, I32, I32, I32, I64,
+                                           P, I64, I32, P]),
+        "mi355_group_rms_norm_f32": (I32, [P, P, P, P, I64, I32, I32, F, I32, P]),
+        "mi355_gated_norm_resid_f32": (I32, [P, P, P, I64, P, P, I64, I32, I32, F, F, I32, P]),
+        "mi355_rms_norm_rows": (I32, [P, P, I64, P, I64, I32, F, I32, P]),
+        "mi355_tanh_rows": (I32, [P, P, I64, I64, I32, I32, P]),
+        "mi355_latent_kv_write": (I32, [P, P, I64, P, P, I32, P, P, I64, I32, I32, I32, F, I32, P]),
+        "mi355_latent_window_attn": (I32, [P, I64, I64, P, I64, I64, P, I64, I32, I32, P, P, I32, P, P, P, P, I64, P, I32,
+                                           I64, I32, I32, I32, I32, I32, F, I32, P]),
+        "mi355_moe_route": (I32, [P, P, P, P, I64, I32, I32, I32, I32, P]),
+        "mi355_moe_sort": (I32, [P, P, P, P, I64, I32, P]),
+        "mi355_moe_gather_rows": (I32, [P, P, P, I64, I32, I32, I32, P]),
+        "mi355_moe_gate_up_rows": (I32, [P, P, P, P, P, I32, I32, I32, I32, I32, P]),
+        "mi355_moe_down_rows": (I32, [P, P, P, P, I32, I32, I32, I32, P]),
+        "mi355_moe_silu_and_mul": (I32, [P, P, I64, I32, I32, P]),
+        "mi355_moe_combine": (I32, [P, P, P, P, I64, I32, I32, I32, P]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
@@ -145,7 +162,11 @@ EXPORTS = ("mi355_abi_version", "mi355_last_error", "mi355_target_arch",
            "mi355_embed_scale_f32", "mi355_resid_add_f32", "mi355_add_rms_norm_f32", "mi355_rms_norm_mix_f32",
            "mi355_gelu_tanh_and_mul", "mi355_gated_head_rms_norm", "mi355_softcap",
            "mi355_rope_partial_kv_write", "mi355_sigmoid_window_attn", "mi355_causal_conv_silu",
-           "mi355_conv_state_update", "mi355_gated_delta_rule", "mi355_gated_delta_rule_workspace")
+           "mi355_conv_state_update", "mi355_gated_delta_rule", "mi355_gated_delta_rule_workspace",
+           "mi355_general_delta_rule", "mi355_general_delta_rule_workspace", "mi355_group_rms_norm_f32",
+           "mi355_gated_norm_resid_f32", "mi355_rms_norm_rows", "mi355_tanh_rows", "mi355_latent_kv_write",
+           "mi355_latent_window_attn", "mi355_moe_route", "mi355_moe_sort", "mi355_moe_gather_rows",
+           "mi355_moe_gate_up_rows", "mi355_moe_down_rows", "mi355_moe_silu_and_mul", "mi355_moe_combine")
 
 
 def check(status: int) -> None:

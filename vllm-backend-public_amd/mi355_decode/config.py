@@ -14,7 +14,7 @@ import os
 from dataclasses import dataclass, field
 from typing import Any, Optional
 
-SUPPORTED_ARCHS = ("LlamaForCausalLM", "Qwen2ForCausalLM", "MistralForCausalLM", "OPTForCausalLM", "Lozupel")
+SUPPORTED_ARCHS = ("LlamaForCausalLM", "Qwen2ForCausalLM", "MistralForCausalLM", "OPTForCausalLM", "Lozupel", "Tativik")
 
 # Well-known geometries, used when --model names one of them and no local
 # config.json exists (synthetic-weight benchmarking; there is no network).
@@ -77,11 +77,58 @@ class DeltaSpec:
 
 
 @dataclass
+class GeneralDeltaSpec:
+    """General delta rule mixer: per head a state [dim, dim] with a decay per key channel (projected
+    through a low-rank pair with a tanh between) and a removal along the unit key at a rate per key
+    channel; receptance, key and value all heads x dim; output normed per head and gated."""
+    heads: int
+    dim: int
+
+
+@dataclass
+class LatentAttnSpec:
+    """Softmax attention through low-rank latents: queries through q_rank, keys and values through
+    kv_rank; per head `dim` unrotated and `rot_dim` rotated query / key coordinates (the rotated key
+    part is one vector shared by all heads, rotation on its first rot_dims coordinates), values of
+    vdim; sliding window; a learned sink per head in the softmax denominator; one output gate per
+    head.  kv_from: the layer whose cached latent and rotated key this layer reads instead of making
+    its own (None: its own)."""
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    kv_rank: int
+    q_rank: int
+    window: int
+    rot_dims: int
+    rot_base: float
+    scale: float
+    kv_from: Optional[int] = None
+
+
+@dataclass
+class MoESpec:
+    """Mixture of experts: `top` of `experts` gated feed-forwards of width ff per token, scored by
+    sigmoid(router), chosen by score + correction inside the best `keep` of `groups` groups of
+    neighbouring experts, weighted by the score itself."""
+    experts: int
+    top: int
+    groups: int
+    keep: int
+    ff: int
+
+
+@dataclass
 class HybridLayerSpec:
-    kind: str                               # "delta": one DeltaSpec; "parallel": window attention beside a delta mixer
+    # "delta": one DeltaSpec; "parallel": window attention beside a delta mixer;
+    # "general_delta": one GeneralDeltaSpec; "latent_attention": one LatentAttnSpec
+    kind: str
     delta: DeltaSpec = None
     attn: Optional[WindowAttnSpec] = None
-    ff: Optional[int] = None                # width of the gated feed-forward, None: the layer has none
+    ff: Optional[int] = None                # width of the dense gated feed-forward, None: the layer has none
+    gdelta: Optional[GeneralDeltaSpec] = None
+    lattn: Optional[LatentAttnSpec] = None
+    moe: Optional[MoESpec] = None           # a mixture-of-experts feed-forward instead of a dense one
 
 
 @dataclass
@@ -96,6 +143,12 @@ class HybridSpec:
     loop_start: int = 0
     loop_stop: int = 0
     loop_times: int = 0                     # 0: no loop
+    # "pre": x += sublayer(norm(x)), norms with one learned number.  "sandwich": the embedding is
+    # normed, and x += residual_mult * norm_b(sublayer(h) * sigmoid(Wg h + bg)) with h = norm(x);
+    # every such norm is an RMS norm in norm_groups equal parts with a weight vector
+    arrangement: str = "pre"
+    norm_groups: int = 1
+    residual_mult: float = 1.0
 
     def runs(self):
         """[(layer index, pass number or None)] in execution order: one cache / state each."""
@@ -106,6 +159,48 @@ class HybridSpec:
         for t in range(self.loop_times):
             out += [(i, t) for i in range(self.loop_start, self.loop_stop)]
         return out + [(i, None) for i in range(self.loop_stop, n)]
+
+    @classmethod
+    def from_tativik(cls, d: dict) -> "HybridSpec":
+        layers = []
+        for i, spec in enumerate(d["layers"]):
+            m, mlp = spec["mixer"], spec.get("mlp")
+            moe = None
+            if mlp is not None:
+                if mlp.get("kind") != "moe":
+                    raise ValueError(f"feed-forward kind {mlp.get('kind')!r} is not supported (moe)")
+                r = mlp["router"]
+                g = r.get("groups") or {"count": 1, "keep": 1}
+                moe = MoESpec(experts=int(r["experts"]), top=int(r["top"]), groups=int(g["count"]), keep=int(g["keep"]),
+                              ff=int(mlp["expert"]["ff"]))
+                if moe.experts % moe.groups or not 1 <= moe.keep <= moe.groups \
+                        or not 1 <= moe.top <= moe.keep * (moe.experts // moe.groups):
+                    raise ValueError(f"layer {i}: {moe.experts} experts in {moe.groups} groups, {moe.keep} kept, "
+                                     f"{moe.top} chosen do not fit")
+            if spec["type"] == "general_delta":
+                layers.append(HybridLayerSpec("general_delta", gdelta=GeneralDeltaSpec(int(m["heads"]), int(m["dim"])),
+                                              moe=moe))
+            elif spec["type"] == "latent_attention":
+                rot = m.get("rot") or {}
+                a = LatentAttnSpec(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
+                                   kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]), window=int(m["mask"]["size"]),
+                                   rot_dims=int(rot.get("dims", m["rot_dim"])), rot_base=float(rot.get("base", 10000.0)),
+                                   scale=float(m["scale"]),
+                                   kv_from=(int(m["kv_from"]) if m.get("kv_from") is not None else None))
+                if a.rot_dims > a.rot_dim or a.rot_dims % 2:
+                    raise ValueError(f"layer {i}: {a.rot_dims} rotated coordinates do not fit rot_dim {a.rot_dim}")
+                if a.kv_from is not None:
+                    src = layers[a.kv_from].lattn if 0 <= a.kv_from < i else None
+                    if src is None or src.kv_from is not None:
+                        raise ValueError(f"layer {i}: kv_from {a.kv_from} must name an earlier latent attention "
+                                         "layer that makes its own latent")
+                    if (src.kv_rank, src.rot_dim, src.rot_dims, src.rot_base) != (a.kv_rank, a.rot_dim, a.rot_dims, a.rot_base):
+                        raise ValueError(f"layer {i}: latent sizes and rotation differ from layer {a.kv_from}'s")
+                layers.append(HybridLayerSpec("latent_attention", lattn=a, moe=moe))
+            else:
+                raise ValueError(f"layer type {spec['type']!r} is not supported (general_delta, latent_attention)")
+        return cls(layers=layers, arrangement="sandwich", norm_groups=int(d["norm"].get("groups", 1)),
+                   residual_mult=float(d.get("residual_mult", 1.0)))
 
     @classmethod
     def from_lozupel(cls, d: dict) -> "HybridSpec":
@@ -184,6 +279,21 @@ class ModelConfig:
                    eos_token_id=d.get("eos_token_id"), family="hybrid", hybrid=spec)
 
     @classmethod
+    def _from_tativik_dict(cls, d: dict) -> "ModelConfig":
+        spec = HybridSpec.from_tativik(d)
+        if int(d["width"]) % spec.norm_groups:
+            raise ValueError(f"width {d['width']} is not a multiple of {spec.norm_groups} norm groups")
+        heads = [m.heads for L in spec.layers for m in (L.gdelta, L.lattn) if m is not None]
+        dims = [L.gdelta.dim if L.gdelta is not None else L.lattn.dim + L.lattn.rot_dim for L in spec.layers]
+        return cls(architecture="Tativik", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]),
+                   intermediate_size=max([L.moe.ff if L.moe else 0 for L in spec.layers] + [0]),
+                   num_hidden_layers=len(spec.layers), num_attention_heads=max(heads), num_key_value_heads=1,
+                   head_dim=max(dims), rope_theta=0.0, rope_scaling=None, rms_norm_eps=float(d["norm"]["eps"]),
+                   max_position_embeddings=int(d.get("max_positions", 1 << 17)), tie_word_embeddings=False,
+                   attention_bias=False, bos_token_id=d.get("bos_token_id"), eos_token_id=d.get("eos_token_id"),
+                   family="hybrid", hybrid=spec)
+
+    @classmethod
     def _from_opt_dict(cls, d: dict) -> "ModelConfig":
         H, nh = d["hidden_size"], d["num_attention_heads"]
         if d.get("word_embed_proj_dim", H) != H:
@@ -217,8 +327,8 @@ class ModelConfig:
             cfg = cls._from_opt_dict(d)
             cfg.torch_dtype = stored
             return cfg
-        if arch == "Lozupel":
-            cfg = cls._from_lozupel_dict(d)
+        if arch in ("Lozupel", "Tativik"):
+            cfg = cls._from_lozupel_dict(d) if arch == "Lozupel" else cls._from_tativik_dict(d)
             cfg.torch_dtype = stored or "bfloat16"
             return cfg
         nh = d["num_attention_heads"]

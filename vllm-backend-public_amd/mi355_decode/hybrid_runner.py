@@ -1,7 +1,12 @@
-"""One model step on one GPU for hybrid decoders (config.HybridSpec; the Lozupel design): every
-layer names its sequence mixer -- a gated delta rule (a linear recurrence with a matrix state per
-head), or a sliding-window attention with sigmoid weights beside such a recurrence -- and may carry a
-gated feed-forward; a span of layers can run several times with shared weights.
+"""One model step on one GPU for hybrid decoders (config.HybridSpec): every layer names its sequence
+mixer and may carry a feed-forward.  Two arrangements share this runner:
+  * "pre" (the Lozupel design): a gated delta rule (a linear recurrence with a matrix state per
+    head), or a sliding-window attention with sigmoid weights beside such a recurrence, and a dense
+    gated feed-forward; a span of layers can run several times with shared weights;
+  * "sandwich" (the Tativik design): a general delta rule (decay per key channel, removal along the
+    unit key) or a softmax attention through low-rank latents (sliding window, a sink in the
+    denominator, latent pages that a later layer may share), then a mixture of experts; every
+    sub-layer sits between a norm in groups and a gated, normed, scaled residual add.
 
 What differs from ModelRunner's decoders, and where it lives:
   * the residual stream is float32 (csrc/resid32.hip: norms with one learned number or a vector,
@@ -104,6 +109,77 @@ class DeltaMixer:
         return r.linear(on, lw.delta_o_w)
 
 
+class GeneralDeltaMixer:
+    """General delta rule with its low-rank decay, removal rate, per-head output norm and gate, on one
+    layer run's state slots."""
+
+    def __init__(self, spec, lw, runner, state_index: int):
+        self.s, self.lw, self.r, self.si = spec, lw, runner, state_index
+
+    def __call__(self, proj: torch.Tensor, b: StepBatch) -> torch.Tensor:
+        s, lw, r = self.s, self.lw, self.r
+        col = lambda n: proj[:, lw.seg[n][0]: lw.seg[n][0] + lw.seg[n][1]]     # noqa: E731
+        decay = r.linear(ops.tanh_rows(col("w1")), lw.w2_w)
+        o = ops.general_delta_rule(col("r"), col("k"), col("v"), decay, lw.w0, col("a"), lw.a_b, r.rec_state[self.si],
+                                   b.cu_seqlens, b.positions, b.state_slots, s.heads, s.dim)
+        return r.linear(ops.gated_head_rms_norm(o, col("g"), lw.head_norm, r.eps, ops.ACT_SIGMOID), lw.o_w)
+
+
+class LatentAttention:
+    """Sliding-window softmax attention through low-rank latents over the latent pages of one layer
+    run -- its own (it writes them first) or those of the layer it shares with."""
+
+    def __init__(self, spec, lw, runner, cache_index: int, writes: bool):
+        self.s, self.lw, self.r, self.ci, self.writes = spec, lw, runner, cache_index, writes
+
+    def __call__(self, proj: torch.Tensor, b: StepBatch) -> torch.Tensor:
+        s, lw, r = self.s, self.lw, self.r
+        col = lambda n: proj[:, lw.seg[n][0]: lw.seg[n][0] + lw.seg[n][1]]     # noqa: E731
+        cache, table = r.latent_cache[self.ci], r.rotary(s.rot_dims, s.rot_base)
+        if self.writes:
+            ops.latent_kv_write(col("dkv"), lw.dkv_norm, table, b.positions, b.slot_mapping, cache, s.kv_rank, s.rot_dim,
+                                r.eps)
+        q = r.linear(ops.rms_norm_rows(col("dq"), lw.dq_norm, r.eps), lw.uq_w)
+        T, hw = q.shape[0], s.dim + s.rot_dim
+        # the unrotated query part of every head into the latent space: the keys then are the cached latents
+        ql = torch.bmm(q.view(T, s.heads, hw)[:, :, : s.dim].transpose(0, 1), lw.uk_w)
+        ol = ops.latent_window_attn(ql, q, hw, s.dim, cache, b.block_tables, b.tok_seq, b.positions, lw.sink, col("g"),
+                                    table, s.window, s.scale)
+        o = torch.bmm(ol, lw.uv_t)                      # [heads, tokens, vdim]
+        return r.linear(o.transpose(0, 1).reshape(T, s.heads * s.vdim), lw.o_w)
+
+
+class MoEFeedForward:
+    """Mixture of experts: fp32 routing, rows sorted by expert, the expert products, the weighted sum."""
+
+    GROUPED_MIN_ROWS = 512          # from this many routed rows on, one library GEMM per expert (needs the counts on the host)
+
+    def __init__(self, spec, lw, runner):
+        self.s, self.lw, self.r = spec, lw, runner
+
+    def __call__(self, h: torch.Tensor) -> torch.Tensor:
+        s, lw = self.s, self.lw
+        T = h.shape[0]
+        ids, wts = ops.moe_route(torch.mm(h.float(), lw.router_w.t()), lw.correction, s.top, s.groups, s.keep)
+        offsets, perm, inv = ops.moe_sort(ids, s.experts)
+        rows = T * s.top
+        if rows >= self.GROUPED_MIN_ROWS and not torch.cuda.is_current_stream_capturing():
+            xs = ops.moe_gather_rows(h, perm, rows, s.top)
+            off = offsets.tolist()
+            gu = torch.empty(rows, 2 * s.ff, dtype=h.dtype, device=h.device)
+            for e in range(s.experts):
+                if off[e + 1] > off[e]:
+                    torch.mm(xs[off[e]: off[e + 1]], lw.gate_up_w[e].t(), out=gu[off[e]: off[e + 1]])
+            act = ops.moe_silu_and_mul(gu)
+            y = torch.empty(rows, h.shape[1], dtype=h.dtype, device=h.device)
+            for e in range(s.experts):
+                if off[e + 1] > off[e]:
+                    torch.mm(act[off[e]: off[e + 1]], lw.down_w[e].t(), out=y[off[e]: off[e + 1]])
+        else:
+            y = ops.moe_down_rows(ops.moe_gate_up_rows(h, lw.gate_up_w, offsets, perm, s.top), lw.down_w, offsets)
+        return ops.moe_combine(y, inv, wts, T, s.top)
+
+
 class HybridRunner(ModelRunner):
     def __init__(self, cfg: ModelConfig, weights: ModelWeights, dtype: torch.dtype, device, num_blocks: int,
                  max_num_seqs: int, max_model_len: int, tp_rank: int = 0, tp_size: int = 1, tp_group=None,
@@ -142,7 +218,25 @@ class HybridRunner(ModelRunner):
         # caches and state, one set per layer RUN (a looped layer: one per pass)
         self.runs = spec.runs()
         self.k_cache, self.v_cache, self.conv_state, self.rec_state, self.mixers = [], [], [], [], []
-        for li, _ in self.runs:
+        self.latent_cache, self.ffs = [], []
+        latent_of = {}                                  # layer index -> index of its latent pages
+        for li, _ in self.runs if spec.arrangement == "sandwich" else ():
+            L, lw = spec.layers[li], weights.layers[li]
+            if L.kind == "general_delta":
+                D = L.gdelta
+                self.rec_state.append(torch.zeros(self.num_state_slots + 1, D.heads, D.dim, D.dim, dtype=torch.float32,
+                                                  device=dev))
+                self.mixers.append(GeneralDeltaMixer(D, lw, self, len(self.rec_state) - 1))
+            else:
+                A = L.lattn
+                if A.kv_from is None:
+                    self.latent_cache.append(torch.zeros(self.num_blocks, BLOCK_SIZE, A.kv_rank + A.rot_dim, dtype=dtype,
+                                                         device=dev))
+                    latent_of[li] = len(self.latent_cache) - 1
+                self.mixers.append(LatentAttention(A, lw, self, latent_of[li if A.kv_from is None else A.kv_from],
+                                                   A.kv_from is None))
+            self.ffs.append(MoEFeedForward(L.moe, lw, self) if L.moe is not None else None)
+        for li, _ in self.runs if spec.arrangement != "sandwich" else ():
             L, lw = spec.layers[li], weights.layers[li]
             D = L.delta
             attn = None
@@ -163,6 +257,7 @@ class HybridRunner(ModelRunner):
         # the samplers want 16-byte aligned logit rows: the head is padded with zero rows to a multiple
         # of 8 and the logits are the first V columns of what it yields
         self.Vp = -(-self.V // 8) * 8
+        self._forward = self._forward_sandwich if spec.arrangement == "sandwich" else self._forward_pre
         self.head_w = weights.lm_head
         if self.Vp != self.V:
             self.head_w = torch.zeros(self.Vp, self.H, dtype=dtype, device=dev)
@@ -206,7 +301,7 @@ class HybridRunner(ModelRunner):
         return {"partial": torch.empty(need, dtype=torch.float32, device=self.device), "num_splits": n}
 
     def kv_cache_bytes_per_block(self) -> int:
-        return sum(t[0].numel() * t.element_size() for t in self.k_cache + self.v_cache)
+        return sum(t[0].numel() * t.element_size() for t in self.k_cache + self.v_cache + self.latent_cache)
 
     def state_bytes_per_slot(self) -> int:
         return sum(t[0].numel() * t.element_size() for t in self.conv_state + self.rec_state)
@@ -221,10 +316,11 @@ class HybridRunner(ModelRunner):
             return
         mats = [self.head_w]
         for lw in self.w.layers:
-            mats += [lw.in_w, lw.delta_o_w, lw.attn_o_w, lw.gate_up_w, lw.down_w, lw.a2_w, lw.g2_w]
+            mats += [getattr(lw, n, None) for n in ("in_w", "delta_o_w", "attn_o_w", "gate_up_w", "down_w", "a2_w", "g2_w",
+                                                    "o_w", "uq_w", "w2_w", "rg2_w")]
         for w in mats:
             # the kernel stages x in 512-wide K slices; narrow outputs leave too few workgroups to pay
-            if w is not None and w.shape[1] % 512 == 0 and w.shape[0] >= 256 and w.shape[0] % 8 == 0:
+            if w is not None and w.dim() == 2 and w.shape[1] % 512 == 0 and w.shape[0] >= 256 and w.shape[0] % 8 == 0:
                 self._tiled_w[w.data_ptr()] = ops.tile_weights(w)
 
     def linear(self, x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -275,7 +371,27 @@ class HybridRunner(ModelRunner):
         return False
 
     # ------------------------------------------------------------------ #
-    def _forward(self, b: StepBatch) -> torch.Tensor:
+    def _forward_sandwich(self, b: StepBatch) -> torch.Tensor:
+        """All layers of the sandwich arrangement over one packed batch; returns the float32 residual
+        stream [tokens, width]."""
+        w, spec = self.w, self.spec
+        G, eps, mult = spec.norm_groups, self.eps, spec.residual_mult
+        resid = ops.embed_scale_f32(w.embed, b.ids, 1.0)
+        ops.group_rms_norm_f32(resid, w.embed_norm, G, eps, out=resid)
+        for ri, (li, _) in enumerate(self.runs):
+            lw = w.layers[li]
+            proj = self.linear(ops.group_rms_norm_f32(resid, lw.norm1, G, eps, dtype=self.dtype), lw.in_w)
+            y = self.mixers[ri](proj, b)
+            gate = proj[:, lw.seg["rg"][0]: lw.seg["rg"][0] + lw.seg["rg"][1]]
+            ops.gated_norm_resid_f32(resid, y, gate, lw.rg1_b, lw.norm1b, G, eps, mult)
+            if self.ffs[ri] is not None:
+                h = ops.group_rms_norm_f32(resid, lw.norm2, G, eps, dtype=self.dtype)
+                ops.gated_norm_resid_f32(resid, self.ffs[ri](h), self.linear(h, lw.rg2_w), lw.rg2_b, lw.norm2b, G, eps, mult)
+            if self.layer_trace is not None:
+                self.layer_trace.append(resid.clone())
+        return resid
+
+    def _forward_pre(self, b: StepBatch) -> torch.Tensor:
         """All layers over one packed batch; returns the float32 residual stream [tokens, width]."""
         w, spec = self.w, self.spec
         resid = ops.embed_scale_f32(w.embed, b.ids, spec.embed_scale)
@@ -308,7 +424,10 @@ class HybridRunner(ModelRunner):
 
     def _logits(self, resid: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Final norm, head and soft cap over the given residual rows."""
-        h = ops.add_rms_norm_f32(resid, self.w.final_norm, self.eps)
+        if self.spec.arrangement == "sandwich":
+            h = ops.group_rms_norm_f32(resid, self.w.final_norm, self.spec.norm_groups, self.eps, dtype=self.dtype)
+        else:
+            h = ops.add_rms_norm_f32(resid, self.w.final_norm, self.eps)
         z = self.linear(h, self.head_w, out=out)
         if self.spec.logit_softcap:
             ops.softcap(z, self.spec.logit_softcap)

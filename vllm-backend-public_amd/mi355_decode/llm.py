@@ -61,8 +61,11 @@ def plan_num_blocks(args: EngineArgs, cfg: ModelConfig, tp_size: int, num_layers
     free memory applies."""
     per_block = 2 * num_layers * (cfg.num_key_value_heads // tp_size) * BLOCK_SIZE * cfg.head_dim * elem_size
     if cfg.family == "hybrid":                        # K and V pages of every layer run that has an attention
-        attn = [cfg.hybrid.layers[i].attn for i, _ in cfg.hybrid.runs() if cfg.hybrid.layers[i].attn is not None]
-        per_block = max(sum(a.kv_heads * (a.dim + a.vdim) for a in attn) * BLOCK_SIZE * elem_size, 1)
+        runs = [cfg.hybrid.layers[i] for i, _ in cfg.hybrid.runs()]
+        per_tok = sum(L.attn.kv_heads * (L.attn.dim + L.attn.vdim) for L in runs if L.attn is not None)
+        # a latent attention caches its latent and one rotated key part, unless it reads another layer's
+        per_tok += sum(L.lattn.kv_rank + L.lattn.rot_dim for L in runs if L.lattn is not None and L.lattn.kv_from is None)
+        per_block = max(per_tok * BLOCK_SIZE * elem_size, 1)
     blocks_per_seq = (max_model_len + BLOCK_SIZE - 1) // BLOCK_SIZE
     want = args.max_num_seqs * blocks_per_seq + 1
     free, total = torch.cuda.mem_get_info(device)

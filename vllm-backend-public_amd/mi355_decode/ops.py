@@ -1035,15 +1035,17 @@ ACT_SILU, ACT_SIGMOID = 0, 1
 def gated_head_rms_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, activation: int,
                         out: torch.Tensor | None = None):
     """o float32 [tokens, heads, dim]; gate [tokens, >= heads * dim] (a column slice is fine);
-    weight float32 [dim].  Returns o / rms(o) * weight * act(gate) as [tokens, heads * dim] in gate's dtype."""
+    weight float32 [dim] (shared by the heads) or [heads * dim].  Returns o / rms(o) * weight * act(gate)
+    as [tokens, heads * dim] in gate's dtype."""
     T, H, D = o.shape
+    wh = H if weight.numel() == H * D and H > 1 else 1
     dt = _dt3(gate, "gate")
     if gate.dim() != 2 or gate.shape[1] != H * D or gate.stride(1) != 1:
         raise ValueError("gate must be [tokens, heads * dim] with a contiguous last dim")
     if out is None:
         out = torch.empty(T, H * D, dtype=gate.dtype, device=o.device)
     check(lib.mi355_gated_head_rms_norm(out.data_ptr(), _f32(o, "o"), gate.data_ptr(), gate.stride(0) if T > 1 else H * D,
-                                        _f32(weight, "weight", D), T, H, D, float(eps), int(activation), dt,
+                                        _f32(weight, "weight", wh * D), wh, T, H, D, float(eps), int(activation), dt,
                                         _stream()))
     return out
 
@@ -1188,4 +1190,209 @@ def gated_delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, beta
         _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(positions, "positions", torch.int64, T),
         _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, num_kv_heads, head_dim, v_dim, T,
         None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), dt, _stream()))
+    return out
+
+
+def general_delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, decay_bias: torch.Tensor,
+                       rate: torch.Tensor, rate_bias: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
+                       positions: torch.Tensor, state_slots: torch.Tensor, num_heads: int, head_dim: int,
+                       out: torch.Tensor | None = None):
+    """The general delta rule over packed chunks: S <- diag(w) S - (a u)(u^T S) + k v^T, o = S^T r with
+    w = exp(-exp(-1/2) sigmoid(decay + decay_bias)), a = sigmoid(rate + rate_bias), u the unit key.
+    r / k / v / decay / rate [tokens, heads * head_dim] (column slices are fine); the biases float32;
+    state float32 [slots, heads, head_dim, head_dim].  Returns o float32 [tokens, heads, head_dim]."""
+    dt = _dt3(r, "r")
+    T, C = r.shape[0], num_heads * head_dim
+    S = cu_seqlens.numel() - 1
+    if tuple(state.shape[1:]) != (num_heads, head_dim, head_dim):
+        raise ValueError("state must be [slots, heads, head_dim, head_dim]")
+    if out is None:
+        out = torch.empty(T, num_heads, head_dim, dtype=torch.float32, device=r.device)
+    if T == 0:
+        return out
+    ws = torch.empty(lib.mi355_general_delta_rule_workspace(T, num_heads, head_dim), dtype=torch.float32, device=r.device)
+    check(lib.mi355_general_delta_rule(
+        _f32(out, "out", T * C), r.data_ptr(), _cols(r, "r", C), _same(k, r, "k"), _cols(k, "k", C), _same(v, r, "v"),
+        _cols(v, "v", C), _same(decay, r, "decay"), _cols(decay, "decay", C), _f32(decay_bias, "decay_bias", C),
+        _same(rate, r, "rate"), _cols(rate, "rate", C), _f32(rate_bias, "rate_bias", C), _f32(state, "state"),
+        _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(positions, "positions", torch.int64, T),
+        _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, head_dim, T, ws.data_ptr(), ws.numel(), dt,
+        _stream()))
+    return out
+
+
+def group_rms_norm_f32(x: torch.Tensor, weight: torch.Tensor, groups: int, eps: float, dtype: torch.dtype | None = None,
+                       out: torch.Tensor | None = None):
+    """RMS norm over each of `groups` equal consecutive parts of the float32 rows x, times weight
+    (float32 [width]).  dtype None: float32 rows (out may be x itself); otherwise activation rows."""
+    T, W = x.shape
+    if out is None:
+        out = torch.empty(T, W, dtype=dtype or torch.float32, device=x.device)
+    if not out.is_contiguous() or out.shape != x.shape or out.dtype != (dtype or torch.float32):
+        raise ValueError("out must be contiguous, shaped like x, in the requested dtype")
+    to32 = dtype is None
+    check(lib.mi355_group_rms_norm_f32(None if to32 else out.data_ptr(), out.data_ptr() if to32 else None, _f32(x, "x"),
+                                       _f32(weight, "weight", W), T, W, int(groups), float(eps),
+                                       _DT[torch.float32] if to32 else _dt3(out, "out"), _stream()))
+    return out
+
+
+def gated_norm_resid_f32(resid: torch.Tensor, y: torch.Tensor, gate: torch.Tensor, bias: torch.Tensor,
+                         weight: torch.Tensor, groups: int, eps: float, mult: float):
+    """resid (float32, in place) += mult * gn(y * sigmoid(gate + bias)) * weight, gn the RMS norm in
+    `groups` parts.  y [tokens, width] contiguous; gate the same shape (a column slice is fine)."""
+    T, W = resid.shape
+    dt = _dt3(y, "y")
+    if y.shape != resid.shape or not y.is_contiguous():
+        raise ValueError("y must be contiguous, shaped like resid")
+    check(lib.mi355_gated_norm_resid_f32(_f32(resid, "resid"), y.data_ptr(), _same(gate, y, "gate"), _cols(gate, "gate", W),
+                                         _f32(bias, "bias", W), _f32(weight, "weight", W), T, W, int(groups), float(eps),
+                                         float(mult), dt, _stream()))
+    return resid
+
+
+def rms_norm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float):
+    """x [rows, n] (a column slice is fine) / rms * weight (float32 [n]) -> contiguous [rows, n] in x's dtype."""
+    dt = _dt3(x, "x")
+    T, n = x.shape
+    out = torch.empty(T, n, dtype=x.dtype, device=x.device)
+    check(lib.mi355_rms_norm_rows(out.data_ptr(), x.data_ptr(), _cols(x, "x", n), _f32(weight, "weight", n), T, n,
+                                  float(eps), dt, _stream()))
+    return out
+
+
+def tanh_rows(x: torch.Tensor):
+    """tanh of x [rows, n] (a column slice is fine) -> contiguous [rows, n]."""
+    dt = _dt3(x, "x")
+    T, n = x.shape
+    out = torch.empty(T, n, dtype=x.dtype, device=x.device)
+    check(lib.mi355_tanh_rows(out.data_ptr(), x.data_ptr(), _cols(x, "x", n), T, n, dt, _stream()))
+    return out
+
+
+def latent_kv_write(x: torch.Tensor, norm_weight: torch.Tensor, cos_sin: torch.Tensor, positions: torch.Tensor,
+                    slot_mapping: torch.Tensor, cache: torch.Tensor, rank: int, rot: int, eps: float):
+    """x [tokens, rank + rot] (a column slice is fine): the first rank columns RMS-normed with norm_weight
+    (float32), the last rot rotated by the table cos_sin [max_pos, rot_dims], both into the row's slot of
+    cache [blocks, 16, rank + rot]."""
+    dt = _dt3(x, "x")
+    T = x.shape[0]
+    if cache.dim() != 3 or tuple(cache.shape[1:]) != (BLOCK_SIZE, rank + rot) or not cache.is_contiguous():
+        raise ValueError("latent pages must be contiguous [blocks, 16, rank + rot]")
+    check(lib.mi355_latent_kv_write(_same(cache, x, "cache"), x.data_ptr(), _cols(x, "x", rank + rot),
+                                    _f32(norm_weight, "norm_weight", rank), _f32(cos_sin, "cos_sin") or x.data_ptr(),
+                                    max(cos_sin.shape[0], 1), _idx(positions, "positions", torch.int64, T),
+                                    _idx(slot_mapping, "slot_mapping", torch.int64, T), T, rank, rot, cos_sin.shape[1],
+                                    float(eps), dt, _stream()))
+
+
+def latent_window_attn(q_latent: torch.Tensor, q: torch.Tensor, q_head_width: int, q_rot_offset: int, cache: torch.Tensor,
+                       block_tables: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor, sink: torch.Tensor,
+                       gate: torch.Tensor | None, cos_sin: torch.Tensor, window: int, scale: float,
+                       out: torch.Tensor | None = None):
+    """Sliding-window softmax attention with a sink over latent pages (see latent_kv_write).  q_latent
+    [heads, tokens, rank]: the unrotated query part multiplied into the latent space; q [tokens, heads *
+    q_head_width] holds the part to rotate at q_rot_offset of every head.  Returns the gated weighted
+    latent [heads, tokens, rank]."""
+    dt = _dt3(q, "q")
+    T = q.shape[0]
+    H, _, rank = q_latent.shape
+    rot = cache.shape[2] - rank
+    if q_latent.shape[1] != T or q_latent.stride(2) != 1:
+        raise ValueError("q_latent must be [heads, tokens, rank] with a contiguous last dim")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be contiguous int32 [chunks, max_blocks]")
+    if cache.dim() != 3 or cache.shape[1] != BLOCK_SIZE or rot < 0 or not cache.is_contiguous():
+        raise ValueError("latent pages must be contiguous [blocks, 16, rank + rot]")
+    if out is None:
+        out = torch.empty(H, T, rank, dtype=q.dtype, device=q.device)
+    if out.shape != q_latent.shape or out.stride(2) != 1 or out.dtype != q.dtype:
+        raise ValueError("out must be shaped like q_latent")
+    check(lib.mi355_latent_window_attn(
+        out.data_ptr(), max(out.stride(1), rank), max(out.stride(0), rank), _same(q_latent, q, "q_latent"),
+        max(q_latent.stride(1), rank), max(q_latent.stride(0), rank), q.data_ptr(), _cols(q, "q", H * q_head_width),
+        q_head_width, q_rot_offset, _same(cache, q, "cache"),
+        block_tables.data_ptr(), block_tables.shape[1], _idx(tok_seq, "tok_seq", torch.int32, T),
+        _idx(positions, "positions", torch.int64, T), _f32(sink, "sink", H),
+        None if gate is None else _same(gate, q, "gate"), 0 if gate is None else _cols(gate, "gate", H),
+        _f32(cos_sin, "cos_sin") or q.data_ptr(), max(cos_sin.shape[0], 1), T, H, rank, rot, cos_sin.shape[1],
+        int(window), float(scale), dt, _stream()))
+    return out
+
+
+def moe_route(logits: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int):
+    """float32 router logits [tokens, experts] -> (ids int32 [tokens, top], weights float32 [tokens, top])."""
+    T, E = logits.shape
+    ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+    wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+    check(lib.mi355_moe_route(ids.data_ptr(), wts.data_ptr(), _f32(logits, "logits"), _f32(correction, "correction", E),
+                              T, E, int(top), int(groups), int(keep), _stream()))
+    return ids, wts
+
+
+def moe_sort(ids: torch.Tensor, experts: int):
+    """Routed rows by expert: (offsets int32 [experts + 1], perm [rows], inv [rows])."""
+    rows = ids.numel()
+    dev = ids.device
+    offsets = torch.empty(experts + 1, dtype=torch.int32, device=dev)
+    perm = torch.empty(max(rows, 1), dtype=torch.int32, device=dev)
+    inv = torch.empty(max(rows, 1), dtype=torch.int32, device=dev)
+    check(lib.mi355_moe_sort(offsets.data_ptr(), perm.data_ptr(), inv.data_ptr(), _idx(ids, "ids", torch.int32), rows,
+                             int(experts), _stream()))
+    return offsets, perm, inv
+
+
+def moe_gather_rows(x: torch.Tensor, perm: torch.Tensor, rows: int, top: int):
+    dt = _dt3(x, "x")
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous")
+    xs = torch.empty(rows, x.shape[1], dtype=x.dtype, device=x.device)
+    check(lib.mi355_moe_gather_rows(xs.data_ptr(), x.data_ptr(), _idx(perm, "perm", torch.int32, rows), rows, int(top),
+                                    x.shape[1], dt, _stream()))
+    return xs
+
+
+def moe_gate_up_rows(x: torch.Tensor, w_gate_up: torch.Tensor, offsets: torch.Tensor, perm: torch.Tensor, top: int):
+    """silu(Wg[e] x) * (Wu[e] x) for every routed row, in expert order: [tokens * top, ff]."""
+    dt = _dt3(x, "x")
+    E, F2, W = w_gate_up.shape
+    if not x.is_contiguous() or x.shape[1] != W or not w_gate_up.is_contiguous():
+        raise ValueError("x must be contiguous [tokens, width], w_gate_up contiguous [experts, 2 ff, width]")
+    rows = x.shape[0] * top
+    act = torch.empty(rows, F2 // 2, dtype=x.dtype, device=x.device)
+    check(lib.mi355_moe_gate_up_rows(act.data_ptr(), x.data_ptr(), _same(w_gate_up, x, "w_gate_up"),
+                                     _idx(offsets, "offsets", torch.int32, E + 1), _idx(perm, "perm", torch.int32, rows),
+                                     E, int(top), W, F2 // 2, dt, _stream()))
+    return act
+
+
+def moe_down_rows(act: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor):
+    dt = _dt3(act, "act")
+    E, W, F = w_down.shape
+    if not act.is_contiguous() or act.shape[1] != F or not w_down.is_contiguous():
+        raise ValueError("act must be contiguous [rows, ff], w_down contiguous [experts, width, ff]")
+    y = torch.empty(act.shape[0], W, dtype=act.dtype, device=act.device)
+    check(lib.mi355_moe_down_rows(y.data_ptr(), act.data_ptr(), _same(w_down, act, "w_down"),
+                                  _idx(offsets, "offsets", torch.int32, E + 1), E, W, F, dt, _stream()))
+    return y
+
+
+def moe_silu_and_mul(x: torch.Tensor):
+    dt = _dt3(x, "x")
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous [rows, 2 ff]")
+    out = torch.empty(x.shape[0], x.shape[1] // 2, dtype=x.dtype, device=x.device)
+    check(lib.mi355_moe_silu_and_mul(out.data_ptr(), x.data_ptr(), x.shape[0], x.shape[1] // 2, dt, _stream()))
+    return out
+
+
+def moe_combine(y: torch.Tensor, inv: torch.Tensor, weights: torch.Tensor, num_tokens: int, top: int):
+    """out[t] = sum_k weights[t, k] * y[inv[t * top + k]]."""
+    dt = _dt3(y, "y")
+    if not y.is_contiguous():
+        raise ValueError("y must be contiguous")
+    out = torch.empty(num_tokens, y.shape[1], dtype=y.dtype, device=y.device)
+    check(lib.mi355_moe_combine(out.data_ptr(), y.data_ptr(), _idx(inv, "inv", torch.int32, num_tokens * top),
+                                _f32(weights, "weights", num_tokens * top), num_tokens, int(top), y.shape[1], dt,
+                                _stream()))
     return out

@@ -103,6 +103,48 @@ class HybridLayerWeights:
 
 
 @dataclass
+class SandwichLayerWeights:
+    """One layer of a hybrid decoder in the "sandwich" arrangement (config.HybridSpec): a general
+    delta rule or a latent attention, then a mixture of experts, each between a norm before and a
+    gated, normed residual after.  Everything that reads the mixer's normed input is ONE matrix in_w
+    (segments `seg`: name -> (first column, width) of the projection's output):
+      general delta:     r | k | v | g | a | w1 | rg    (w1: the low-rank input of the decay, widened by w2_w)
+      latent attention:  dq | dkv | g | rg              (dkv only if the layer makes its own latent)
+    rg is the residual gate of the sub-layer.  Norm weights, biases, sinks, the router and its
+    correction are float32; expert matrices are stacked [experts, ...]."""
+    norm1: torch.Tensor                     # f32 [width] each
+    norm1b: torch.Tensor
+    in_w: torch.Tensor
+    seg: dict
+    rg1_b: torch.Tensor                     # f32 [width]
+    o_w: torch.Tensor                       # [width, heads * dim] / [width, heads * vdim]
+    # general delta rule
+    w2_w: Optional[torch.Tensor] = None     # [heads * dim, rank]
+    w0: Optional[torch.Tensor] = None       # f32 [heads * dim]
+    a_b: Optional[torch.Tensor] = None      # f32 [heads * dim]
+    head_norm: Optional[torch.Tensor] = None    # f32 [heads * dim]
+    # latent attention
+    dq_norm: Optional[torch.Tensor] = None  # f32 [q_rank]
+    uq_w: Optional[torch.Tensor] = None     # [heads * (dim + rot_dim), q_rank]
+    dkv_norm: Optional[torch.Tensor] = None     # f32 [kv_rank]
+    uk_w: Optional[torch.Tensor] = None     # [heads, dim, kv_rank]
+    uv_t: Optional[torch.Tensor] = None     # [heads, kv_rank, vdim]: the value up-projection, transposed per head
+    sink: Optional[torch.Tensor] = None     # f32 [heads]
+    # mixture of experts
+    norm2: Optional[torch.Tensor] = None
+    norm2b: Optional[torch.Tensor] = None
+    rg2_w: Optional[torch.Tensor] = None    # [width, width]
+    rg2_b: Optional[torch.Tensor] = None    # f32 [width]
+    router_w: Optional[torch.Tensor] = None     # f32 [experts, width]
+    correction: Optional[torch.Tensor] = None   # f32 [experts]
+    gate_up_w: Optional[torch.Tensor] = None    # [experts, 2 ff, width]
+    down_w: Optional[torch.Tensor] = None       # [experts, width, ff]
+
+    def tensors(self):
+        return [t for t in vars(self).values() if isinstance(t, torch.Tensor)]
+
+
+@dataclass
 class ModelWeights:
     embed: torch.Tensor
     layers: list = field(default_factory=list)
@@ -112,17 +154,18 @@ class ModelWeights:
     pos_embed: Optional[torch.Tensor] = None     # learned positions (OPT): [max_positions + offset, hidden]
     final_norm_b: Optional[torch.Tensor] = None
     loop_step: Optional[torch.Tensor] = None     # hybrid decoders with a loop: [passes, width]
+    embed_norm: Optional[torch.Tensor] = None    # hybrid decoders that norm the embedding: f32 [width]
 
     def nbytes(self) -> int:
         total = self.embed.numel() * self.embed.element_size()
         if self.lm_head.untyped_storage().data_ptr() != self.embed.untyped_storage().data_ptr():
             total += self.lm_head.numel() * self.lm_head.element_size()
         total += self.final_norm.numel() * self.final_norm.element_size()
-        for t in (self.pos_embed, self.final_norm_b, self.loop_step):
+        for t in (self.pos_embed, self.final_norm_b, self.loop_step, self.embed_norm):
             if t is not None:
                 total += t.numel() * t.element_size()
         for lw in self.layers:
-            ts = lw.tensors() if isinstance(lw, (OPTLayerWeights, HybridLayerWeights)) else \
+            ts = lw.tensors() if isinstance(lw, (OPTLayerWeights, HybridLayerWeights, SandwichLayerWeights)) else \
                 (lw.qkv_w, lw.qkv_b, lw.o_w, lw.gate_up_w, lw.down_w, lw.input_norm, lw.post_norm)
             for t in ts:
                 if t is not None:
@@ -276,6 +319,8 @@ def _hybrid_from_getter(cfg: ModelConfig, get, dtype, device, tp_size: int, num_
     _hybrid_one_gpu(tp_size, num_layers)
     spec = cfg.hybrid
     W = cfg.hidden_size
+    if spec.arrangement == "sandwich":
+        return _sandwich_from_getter(cfg, get, dtype, device)
 
     def put(t, dt=dtype):
         return t.to(dt).contiguous().to(device)
@@ -350,11 +395,136 @@ def _hybrid_from_getter(cfg: ModelConfig, get, dtype, device, tp_size: int, num_
     return w
 
 
+def _fuse_segments(parts, W: int, put):
+    """One matrix of all the projections that read the same input; every segment starts on a 16-byte
+    boundary of the output row.  Returns (matrix, {name: (first column, width)})."""
+    seg, at = {}, 0
+    for name, t in parts:
+        if t.dim() != 2 or t.shape[1] != W:
+            raise ValueError(f"segment {name}: shape {tuple(t.shape)}, expected [*, {W}]")
+        seg[name] = (at, int(t.shape[0]))
+        at += -(-int(t.shape[0]) // 8) * 8
+    full = torch.zeros(at, W, dtype=parts[0][1].dtype)
+    for name, t in parts:
+        full[seg[name][0]: seg[name][0] + seg[name][1]] = t
+    return put(full), seg
+
+
+def _sandwich_from_getter(cfg: ModelConfig, get, dtype, device) -> ModelWeights:
+    """Tativik checkpoints: 'embed', 'embed.norm', 'final.norm', 'head', and per layer i 'l<i>.norm1|norm1b|
+    norm2|norm2b', 'l<i>.rg1|rg2' with '.b', 'l<i>.mix.*' (general delta: r k v g a a.b w1 w2 w0 norm o;
+    latent attention: dq dq.norm uq [dkv dkv.norm] uk uv sink g o), 'l<i>.mlp.router|correction' and
+    'l<i>.mlp.e<j>.gate|up|down'.  Linear weights are [out, in]."""
+    spec, W = cfg.hybrid, cfg.hidden_size
+
+    def put(t, dt=dtype):
+        return t.to(dt).contiguous().to(device)
+
+    def f32(t):
+        return put(t.reshape(-1), torch.float32)
+
+    def expect(name, shape):
+        t = get(name)
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t
+
+    w = ModelWeights(embed=put(expect("embed", (cfg.vocab_size, W))), embed_norm=f32(expect("embed.norm", (W,))))
+    for i, L in enumerate(spec.layers):
+        p, m = f"l{i}.", f"l{i}.mix."
+        kw = dict(norm1=f32(expect(p + "norm1", (W,))), norm1b=f32(expect(p + "norm1b", (W,))),
+                  rg1_b=f32(expect(p + "rg1.b", (W,))))
+        rg1 = ("rg", expect(p + "rg1", (W, W)))
+        if L.kind == "general_delta":
+            D = L.gdelta
+            C = D.heads * D.dim
+            w1 = get(m + "w1")
+            in_w, seg = _fuse_segments([(n, expect(m + n, (C, W))) for n in "rkvga"] + [("w1", w1), rg1], W, put)
+            kw.update(in_w=in_w, seg=seg, o_w=put(expect(m + "o", (W, C))), w2_w=put(expect(m + "w2", (C, w1.shape[0]))),
+                      w0=f32(expect(m + "w0", (C,))), a_b=f32(expect(m + "a.b", (C,))),
+                      head_norm=f32(expect(m + "norm", (C,))))
+        else:
+            A = L.lattn
+            parts = [("dq", expect(m + "dq", (A.q_rank, W)))]
+            if A.kv_from is None:
+                parts.append(("dkv", expect(m + "dkv", (A.kv_rank + A.rot_dim, W))))
+                kw["dkv_norm"] = f32(expect(m + "dkv.norm", (A.kv_rank,)))
+            in_w, seg = _fuse_segments(parts + [("g", expect(m + "g", (A.heads, W))), rg1], W, put)
+            uv = expect(m + "uv", (A.heads * A.vdim, A.kv_rank)).view(A.heads, A.vdim, A.kv_rank)
+            kw.update(in_w=in_w, seg=seg, o_w=put(expect(m + "o", (W, A.heads * A.vdim))),
+                      dq_norm=f32(expect(m + "dq.norm", (A.q_rank,))),
+                      uq_w=put(expect(m + "uq", (A.heads * (A.dim + A.rot_dim), A.q_rank))),
+                      uk_w=put(expect(m + "uk", (A.heads * A.dim, A.kv_rank)).view(A.heads, A.dim, A.kv_rank)),
+                      uv_t=put(uv.transpose(1, 2)), sink=f32(expect(m + "sink", (A.heads,))))
+        if L.moe is not None:
+            M, q = L.moe, p + "mlp."
+            gu = torch.stack([torch.cat([expect(f"{q}e{e}.gate", (M.ff, W)), expect(f"{q}e{e}.up", (M.ff, W))], dim=0)
+                              for e in range(M.experts)])
+            kw.update(norm2=f32(expect(p + "norm2", (W,))), norm2b=f32(expect(p + "norm2b", (W,))),
+                      rg2_w=put(expect(p + "rg2", (W, W))), rg2_b=f32(expect(p + "rg2.b", (W,))),
+                      router_w=put(expect(q + "router", (M.experts, W)), torch.float32),
+                      correction=f32(expect(q + "correction", (M.experts,))), gate_up_w=put(gu),
+                      down_w=put(torch.stack([expect(f"{q}e{e}.down", (W, M.ff)) for e in range(M.experts)])))
+        w.layers.append(SandwichLayerWeights(**kw))
+    w.final_norm = f32(expect("final.norm", (W,)))
+    w.lm_head = put(expect("head", (cfg.vocab_size, W)))
+    return w
+
+
+def sandwich_synthetic_state(cfg: ModelConfig, seed: int = 0, decay_rank: int = 64, device="cpu",
+                             dtype=torch.float32) -> dict:
+    """Seeded random tensors under a Tativik checkpoint's names (benchmarks and tests: nothing can be
+    downloaded).  `decay_rank`: the inner width of the low-rank decay projection."""
+    spec, W = cfg.hybrid, cfg.hidden_size
+    gen = torch.Generator(device=device).manual_seed(seed)
+
+    def mat(*shape, s=1.0):
+        return torch.empty(shape, dtype=dtype, device=device).normal_(0.0, s, generator=gen)
+
+    def near(value, *shape, s=0.1):
+        return torch.full(shape, float(value), dtype=dtype, device=device) + mat(*shape, s=s)
+
+    st = {"embed": mat(cfg.vocab_size, W), "embed.norm": near(1.0, W), "head": mat(cfg.vocab_size, W, s=W ** -0.5),
+          "final.norm": near(1.0, W)}
+    for i, L in enumerate(spec.layers):
+        p, m = f"l{i}.", f"l{i}.mix."
+        st[p + "norm1"], st[p + "norm1b"] = near(1.0, W), near(1.0, W)
+        st[p + "rg1"], st[p + "rg1.b"] = mat(W, W, s=W ** -0.5), mat(W, s=0.5)
+        if L.kind == "general_delta":
+            C = L.gdelta.heads * L.gdelta.dim
+            for n in "rkvga":
+                st[m + n] = mat(C, W, s=W ** -0.5)
+            st[m + "a.b"], st[m + "w0"], st[m + "norm"] = mat(C, s=0.5), mat(C), near(1.0, C)
+            st[m + "w1"], st[m + "w2"] = mat(decay_rank, W, s=W ** -0.5), mat(C, decay_rank, s=decay_rank ** -0.5)
+            st[m + "o"] = mat(W, C, s=C ** -0.5)
+        else:
+            A = L.lattn
+            st[m + "dq"], st[m + "dq.norm"] = mat(A.q_rank, W, s=W ** -0.5), near(1.0, A.q_rank)
+            st[m + "uq"] = mat(A.heads * (A.dim + A.rot_dim), A.q_rank, s=A.q_rank ** -0.5)
+            if A.kv_from is None:
+                st[m + "dkv"], st[m + "dkv.norm"] = mat(A.kv_rank + A.rot_dim, W, s=W ** -0.5), near(1.0, A.kv_rank)
+            st[m + "uk"] = mat(A.heads * A.dim, A.kv_rank, s=A.kv_rank ** -0.5)
+            st[m + "uv"] = mat(A.heads * A.vdim, A.kv_rank, s=A.kv_rank ** -0.5)
+            st[m + "sink"], st[m + "g"] = mat(A.heads), mat(A.heads, W, s=W ** -0.5)
+            st[m + "o"] = mat(W, A.heads * A.vdim, s=(A.heads * A.vdim) ** -0.5)
+        if L.moe is not None:
+            M, q = L.moe, p + "mlp."
+            st[p + "norm2"], st[p + "norm2b"] = near(1.0, W), near(1.0, W)
+            st[p + "rg2"], st[p + "rg2.b"] = mat(W, W, s=W ** -0.5), mat(W, s=0.5)
+            st[q + "router"], st[q + "correction"] = mat(M.experts, W, s=W ** -0.5), mat(M.experts, s=0.3)
+            for e in range(M.experts):
+                st[f"{q}e{e}.gate"], st[f"{q}e{e}.up"] = mat(M.ff, W, s=W ** -0.5), mat(M.ff, W, s=W ** -0.5)
+                st[f"{q}e{e}.down"] = mat(W, M.ff, s=M.ff ** -0.5)
+    return st
+
+
 def hybrid_synthetic_state(cfg: ModelConfig, seed: int = 0, std: float = 0.02, rank: int = 32, device="cpu",
                            dtype=torch.float32) -> dict:
     """Seeded random tensors under a Lozupel checkpoint's names (benchmarks and tests: nothing can be
     downloaded).  `rank`: the inner width of the low-rank decay / gate projections."""
     spec, W = cfg.hybrid, cfg.hidden_size
+    if spec.arrangement == "sandwich":
+        return sandwich_synthetic_state(cfg, seed=seed, device=device, dtype=dtype)
     gen = torch.Generator(device=device).manual_seed(seed)
 
     def mat(*shape, s=std):
