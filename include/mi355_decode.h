@@ -846,6 +846,8 @@ int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t stride, int32_
  * r / k / v / decay / rate are [tokens, heads * head_dim] activations (column slices are fine), the
  * biases fp32 [heads * head_dim]; everything past the projections is fp32.  o is fp32
  * [tokens, heads, head_dim].  workspace: mi355_general_delta_rule_workspace(...) floats.
+ * long_chunks 1: state rows split over adjacent lanes (chunks of many tokens); 0: one state column
+ * per lane (chunks of a token or two: decode).  Both give the same numbers for any chunk.
  */
 int64_t mi355_general_delta_rule_workspace(int64_t num_tokens, int32_t num_heads, int32_t head_dim);
 int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_stride, const void* k,
@@ -854,8 +856,9 @@ int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_stride, cons
                                  int64_t rate_stride, const float* rate_bias, float* state,
                                  const int32_t* cu_seqlens, const int64_t* positions,
                                  const int32_t* state_slots, int32_t num_seqs, int32_t num_heads,
-                                 int32_t head_dim, int64_t num_tokens, float* workspace,
-                                 int64_t workspace_floats, int32_t dtype, void* stream);
+                                 int32_t head_dim, int64_t num_tokens, int32_t long_chunks,
+                                 float* workspace, int64_t workspace_floats, int32_t dtype,
+                                 void* stream);
 
 /*
  * More kernels on the fp32 residual stream.  gn(x): an RMS norm taken separately over each of

@@ -142,7 +142,7 @@ def test_group_norms_and_the_gated_residual(dtype, groups):
     assert (out.float().cpu() - ref).abs().max() <= tol * ref.abs().max()
 
 
-def _gdelta_in_cuts(x, w0, ab, cuts, H, d, slot=2, slots=4):
+def _gdelta_in_cuts(x, w0, ab, cuts, H, d, slot=2, slots=4, long_chunks=True):
     """x [T, 5, H * d] = r | k | v | decay | rate inputs of one sequence fed in portions."""
     from mi355_decode import ops
     state = torch.full((slots, H, d, d), float("nan"), device="cuda")
@@ -154,7 +154,8 @@ def _gdelta_in_cuts(x, w0, ab, cuts, H, d, slot=2, slots=4):
                                            xs[:, 4 * C:], ab.cuda(), state,
                                            torch.tensor([0, n], dtype=torch.int32, device="cuda"),
                                            torch.arange(at, at + n, dtype=torch.int64, device="cuda"),
-                                           torch.tensor([slot], dtype=torch.int32, device="cuda"), H, d).cpu())
+                                           torch.tensor([slot], dtype=torch.int32, device="cuda"), H, d,
+                                           long_chunks=long_chunks).cpu())
         at += n
     return torch.cat(outs), state
 
@@ -174,8 +175,9 @@ def test_general_delta_rule_whole_portions_and_single_tokens(H, d):
     w0, ab = torch.randn(H * d, generator=g), torch.randn(H * d, generator=g) * 0.5
     ref = _gdelta_ref(x, w0, ab, H, d)
     for cuts in ([T], [1] * T, [2, 3, 1, 17, 2, 16]):
-        got, _ = _gdelta_in_cuts(x, w0, ab, cuts, H, d)
-        assert (got - ref).abs().max() <= 3e-5 * ref.abs().max(), cuts
+        for long_chunks in (True, False):                   # state rows split over lanes; one state column per lane
+            got, _ = _gdelta_in_cuts(x, w0, ab, cuts, H, d, long_chunks=long_chunks)
+            assert (got - ref).abs().max() <= 3e-5 * ref.abs().max(), (cuts, long_chunks)
 
 
 def test_general_delta_rule_keeps_a_far_write_removes_it_along_its_key_and_forgets_it_with_decay():

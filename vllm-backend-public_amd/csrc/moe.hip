@@ -113,52 +113,109 @@ __global__ __launch_bounds__(256) void moe_gather_rows_kernel(typename Elem<T>::
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
+// Rows of an expert are taken kRowBlock at a time, so that a weight element is loaded once per block
+// of rows and not once per row.
+constexpr int kRowBlock = 8;
+
+// dot products of one weight row w [n] with up to kRowBlock rows xr[r] [n]; every lane of the wave gets the sums
+template <typename T, bool VEC>
+__device__ __forceinline__ void rows_dot(const typename Elem<T>::S* wbase, const typename Elem<T>::S* w,
+                                         const typename Elem<T>::S* xbase, const typename Elem<T>::S* const (&xr)[kRowBlock],
+                                         int n, int lane, float (&acc)[kRowBlock]) {
+#pragma unroll
+  for (int r = 0; r < kRowBlock; ++r) acc[r] = 0.f;
+  if constexpr (VEC) {                                  // 16-bit storage, n a multiple of 8, 16-byte aligned rows
+    for (int c = lane * 8; c < n; c += 512) {
+      float wv[8];
+      unpack8<T>(MI355_LD(uint4, wbase, reinterpret_cast<const uint16_t*>(w) + c), wv);
+#pragma unroll
+      for (int r = 0; r < kRowBlock; ++r) {
+        float xv[8];
+        unpack8<T>(MI355_LD(uint4, xbase, reinterpret_cast<const uint16_t*>(xr[r]) + c), xv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[r] += wv[i] * xv[i];
+      }
+    }
+  } else {
+    for (int c = lane; c < n; c += 64) {
+      const float wv = MI355_LDF(T, wbase, w + c);
+#pragma unroll
+      for (int r = 0; r < kRowBlock; ++r) acc[r] += wv * MI355_LDF(T, xbase, xr[r] + c);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < kRowBlock; ++r) acc[r] = wave_sum(acc[r]);
+}
+
+template <typename T, bool VEC> struct RowsDot {
+  static __device__ __forceinline__ void run(const typename Elem<T>::S* wbase, const typename Elem<T>::S* w,
+                                             const typename Elem<T>::S* xbase,
+                                             const typename Elem<T>::S* const (&xr)[kRowBlock], int n, int lane,
+                                             float (&acc)[kRowBlock]) {
+    rows_dot<T, VEC>(wbase, w, xbase, xr, n, lane, acc);
+  }
+};
+template <> struct RowsDot<F32, true> {                  // (never selected: 32-bit storage takes the scalar form)
+  static __device__ __forceinline__ void run(const float* wbase, const float* w, const float* xbase,
+                                             const float* const (&xr)[kRowBlock], int n, int lane, float (&acc)[kRowBlock]) {
+    rows_dot<F32, false>(wbase, w, xbase, xr, n, lane, acc);
+  }
+};
+
 // one wave per (expert, hidden unit f): gate and up rows of that unit against every row routed to the expert
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(typename Elem<T>::S* __restrict__ a,
                                                                const typename Elem<T>::S* __restrict__ x,
                                                                const typename Elem<T>::S* __restrict__ w_gate_up,
                                                                const int32_t* __restrict__ offsets,
                                                                const int32_t* __restrict__ perm, int top, int W, int F) {
+  typedef typename Elem<T>::S E;
   const int e = blockIdx.y, lane = threadIdx.x & 63;
   const int f = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (f >= F) return;
   const int lo = MI355_LD(int32_t, offsets, offsets + e), hi = MI355_LD(int32_t, offsets, offsets + e + 1);
-  const typename Elem<T>::S* wg = w_gate_up + (static_cast<int64_t>(e) * 2 * F + f) * W;
-  const typename Elem<T>::S* wu = wg + static_cast<int64_t>(F) * W;
-  for (int p = lo; p < hi; ++p) {
-    const int64_t t = MI355_LD(int32_t, perm, perm + p) / top;
-    float g = 0.f, u = 0.f;
-    for (int c = lane; c < W; c += 64) {
-      const float xv = MI355_LDF(T, x, x + t * W + c);
-      g += xv * MI355_LDF(T, w_gate_up, wg + c);
-      u += xv * MI355_LDF(T, w_gate_up, wu + c);
+  const E* wg = w_gate_up + (static_cast<int64_t>(e) * 2 * F + f) * W;
+  const E* wu = wg + static_cast<int64_t>(F) * W;
+  for (int p0 = lo; p0 < hi; p0 += kRowBlock) {
+    const E* xr[kRowBlock];
+#pragma unroll
+    for (int r = 0; r < kRowBlock; ++r) {                // rows past the expert's last: the block's first row again, not stored
+      const int p = p0 + r < hi ? p0 + r : p0;
+      xr[r] = x + static_cast<int64_t>(MI355_LD(int32_t, perm, perm + p) / top) * W;
     }
-    g = wave_sum(g);
-    u = wave_sum(u);
-    if (lane == 0) {
-      const float gr = elem_to_f<T>(elem_from_f<T>(g)), ur = elem_to_f<T>(elem_from_f<T>(u));   // as stored by a product
-      MI355_STF(T, a, a + static_cast<int64_t>(p) * F + f, silu_f(gr) * ur);
+    float g[kRowBlock], u[kRowBlock];
+    RowsDot<T, VEC>::run(w_gate_up, wg, x, xr, W, lane, g);
+    RowsDot<T, VEC>::run(w_gate_up, wu, x, xr, W, lane, u);
+#pragma unroll
+    for (int r = 0; r < kRowBlock; ++r) {
+      if (lane == r && p0 + r < hi) {
+        const float gr = elem_to_f<T>(elem_from_f<T>(g[r])), ur = elem_to_f<T>(elem_from_f<T>(u[r]));   // as stored by a product
+        MI355_STF(T, a, a + static_cast<int64_t>(p0 + r) * F + f, silu_f(gr) * ur);
+      }
     }
   }
 }
 
-template <typename T>
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void moe_down_rows_kernel(typename Elem<T>::S* __restrict__ y,
                                                             const typename Elem<T>::S* __restrict__ a,
                                                             const typename Elem<T>::S* __restrict__ w_down,
                                                             const int32_t* __restrict__ offsets, int W, int F) {
+  typedef typename Elem<T>::S E;
   const int e = blockIdx.y, lane = threadIdx.x & 63;
   const int c = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (c >= W) return;
   const int lo = MI355_LD(int32_t, offsets, offsets + e), hi = MI355_LD(int32_t, offsets, offsets + e + 1);
-  const typename Elem<T>::S* wd = w_down + (static_cast<int64_t>(e) * W + c) * F;
-  for (int p = lo; p < hi; ++p) {
-    float s = 0.f;
-    for (int f = lane; f < F; f += 64)
-      s += MI355_LDF(T, a, a + static_cast<int64_t>(p) * F + f) * MI355_LDF(T, w_down, wd + f);
-    s = wave_sum(s);
-    if (lane == 0) MI355_STF(T, y, y + static_cast<int64_t>(p) * W + c, s);
+  const E* wd = w_down + (static_cast<int64_t>(e) * W + c) * F;
+  for (int p0 = lo; p0 < hi; p0 += kRowBlock) {
+    const E* ar[kRowBlock];
+#pragma unroll
+    for (int r = 0; r < kRowBlock; ++r) ar[r] = a + static_cast<int64_t>(p0 + r < hi ? p0 + r : p0) * F;
+    float s[kRowBlock];
+    RowsDot<T, VEC>::run(w_down, wd, a, ar, F, lane, s);
+#pragma unroll
+    for (int r = 0; r < kRowBlock; ++r)
+      if (lane == r && p0 + r < hi) MI355_STF(T, y, y + static_cast<int64_t>(p0 + r) * W + c, s[r]);
   }
 }
 
@@ -246,10 +303,17 @@ extern "C" int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* 
   REQ_DTYPE(dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>((ff + 3) / 4), static_cast<unsigned>(experts));
-  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_gate_up_rows_kernel<TT>), grid, dim3(256), 0, s,
-                                                  static_cast<Elem<TT>::S*>(act), static_cast<const Elem<TT>::S*>(x),
-                                                  static_cast<const Elem<TT>::S*>(w_gate_up), offsets, perm, top, width,
-                                                  ff));
+  const bool vec = dtype != MI355_F32 && width % 8 == 0 && aligned16(x) && aligned16(w_gate_up);
+  MI355_DISPATCH_DTYPE3(dtype, {
+    if (vec)
+      hipLaunchKernelGGL((moe_gate_up_rows_kernel<TT, true>), grid, dim3(256), 0, s, static_cast<Elem<TT>::S*>(act),
+                         static_cast<const Elem<TT>::S*>(x), static_cast<const Elem<TT>::S*>(w_gate_up), offsets, perm, top,
+                         width, ff);
+    else
+      hipLaunchKernelGGL((moe_gate_up_rows_kernel<TT, false>), grid, dim3(256), 0, s, static_cast<Elem<TT>::S*>(act),
+                         static_cast<const Elem<TT>::S*>(x), static_cast<const Elem<TT>::S*>(w_gate_up), offsets, perm, top,
+                         width, ff);
+  });
   return check_launch("moe_gate_up_rows");
 }
 
@@ -260,9 +324,15 @@ extern "C" int32_t mi355_moe_down_rows(void* y, const void* act, const void* w_d
   REQ_DTYPE(dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>((width + 3) / 4), static_cast<unsigned>(experts));
-  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_down_rows_kernel<TT>), grid, dim3(256), 0, s,
-                                                  static_cast<Elem<TT>::S*>(y), static_cast<const Elem<TT>::S*>(act),
-                                                  static_cast<const Elem<TT>::S*>(w_down), offsets, width, ff));
+  const bool vec = dtype != MI355_F32 && ff % 8 == 0 && aligned16(act) && aligned16(w_down);
+  MI355_DISPATCH_DTYPE3(dtype, {
+    if (vec)
+      hipLaunchKernelGGL((moe_down_rows_kernel<TT, true>), grid, dim3(256), 0, s, static_cast<Elem<TT>::S*>(y),
+                         static_cast<const Elem<TT>::S*>(act), static_cast<const Elem<TT>::S*>(w_down), offsets, width, ff);
+    else
+      hipLaunchKernelGGL((moe_down_rows_kernel<TT, false>), grid, dim3(256), 0, s, static_cast<Elem<TT>::S*>(y),
+                         static_cast<const Elem<TT>::S*>(act), static_cast<const Elem<TT>::S*>(w_down), offsets, width, ff);
+  });
   return check_launch("moe_down_rows");
 }
 

@@ -744,6 +744,53 @@ __global__ __launch_bounds__(64) void general_delta_rule_kernel(
   }
 }
 
+// The same recurrence for chunks of one or two tokens (decode): one wave per (chunk, head, 64 value
+// channels), lane j owns column j of S in registers, so a state row is one coalesced load; the
+// per-token vectors come from the prepared rows (every lane reads the same address).
+template <typename T, int D>
+__global__ __launch_bounds__(64) void general_delta_rule_cols_kernel(
+    float* __restrict__ o, const typename Elem<T>::S* __restrict__ v, int64_t v_stride, const float* __restrict__ ws,
+    int dp, float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int64_t* __restrict__ positions,
+    const int32_t* __restrict__ state_slots, int H, int d) {
+  const int s = blockIdx.x, h = blockIdx.y, col = blockIdx.z * 64 + threadIdx.x;
+  const int64_t cs = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s);
+  const int64_t n = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1) - cs;
+  if (n <= 0) return;
+  const int64_t slot = MI355_LD(int32_t, state_slots, state_slots + s);
+  float* sp = state + ((slot * H + h) * d) * d;
+  const bool live = col < d;
+  const bool fresh = MI355_LD(int64_t, positions, positions + cs) == 0;
+  float S[D];
+#pragma unroll
+  for (int i = 0; i < D; ++i) S[i] = (live && !fresh && i < d) ? MI355_LD(float, state, sp + static_cast<int64_t>(i) * d + col) : 0.f;
+  for (int64_t t = cs; t < cs + n; ++t) {
+    const float* p = ws + (t * H + h) * 5 * dp;
+    const float vj = live ? MI355_LDF(T, v, v + t * v_stride + static_cast<int64_t>(h) * d + col) : 0.f;
+    float d0 = 0.f, d1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < D; i += 2) {
+      d0 += S[i] * MI355_LD(float, ws, p + dp + i);
+      d1 += S[i + 1] * MI355_LD(float, ws, p + dp + i + 1);
+    }
+    const float dot = d0 + d1;
+    float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < D; i += 2) {
+      S[i] = MI355_LD(float, ws, p + i) * S[i] - MI355_LD(float, ws, p + 2 * dp + i) * dot + MI355_LD(float, ws, p + 3 * dp + i) * vj;
+      S[i + 1] = MI355_LD(float, ws, p + i + 1) * S[i + 1] - MI355_LD(float, ws, p + 2 * dp + i + 1) * dot +
+                 MI355_LD(float, ws, p + 3 * dp + i + 1) * vj;
+      o0 += S[i] * MI355_LD(float, ws, p + 4 * dp + i);
+      o1 += S[i + 1] * MI355_LD(float, ws, p + 4 * dp + i + 1);
+    }
+    if (live) MI355_ST(float, o, o + (t * H + h) * d + col, o0 + o1);
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < D; ++i)
+      if (i < d) MI355_ST(float, state, sp + static_cast<int64_t>(i) * d + col, S[i]);
+  }
+}
+
 // out = sigmoid(gate) * sum of the key-range partial sums of sigmoid_window_attn_mfma_kernel
 template <typename T>
 __global__ __launch_bounds__(256) void window_attn_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial,
@@ -1023,8 +1070,8 @@ extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_s
                                             const float* decay_bias, const void* rate, int64_t rate_stride,
                                             const float* rate_bias, float* state, const int32_t* cu_seqlens,
                                             const int64_t* positions, const int32_t* state_slots, int32_t num_seqs,
-                                            int32_t num_heads, int32_t head_dim, int64_t num_tokens, float* workspace,
-                                            int64_t workspace_floats, int32_t dtype, void* stream) {
+                                            int32_t num_heads, int32_t head_dim, int64_t num_tokens, int32_t long_chunks,
+                                            float* workspace, int64_t workspace_floats, int32_t dtype, void* stream) {
   MI355_REQUIRE(o && r && k && v && decay && decay_bias && rate && rate_bias && state && cu_seqlens && positions &&
                     state_slots && workspace,
                 MI355_ERR_INVALID, "general_delta_rule: null pointer");
@@ -1048,6 +1095,12 @@ extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_s
   const dim3 pgrid(static_cast<unsigned>(num_tokens), static_cast<unsigned>(num_heads));
   const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads),
                   static_cast<unsigned>((head_dim + cols - 1) / cols));
+  // the form for chunks of a token or two: one state column per lane
+  const dim3 cgrid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>((head_dim + 63) / 64));
+#define MI355_GCOLS(D)                                                                                                 \
+  hipLaunchKernelGGL((general_delta_rule_cols_kernel<TT, D>), cgrid, dim3(64), 0, s, o, static_cast<const E*>(v),     \
+                     v_stride, workspace, static_cast<int>(dp), state, cu_seqlens, positions, state_slots, num_heads, \
+                     head_dim)
 #define MI355_GDELTA(TT, R, DR, PF)                                                                                  \
   hipLaunchKernelGGL((general_delta_rule_kernel<TT, R, DR, PF>), grid, dim3(64), 0, s, o,                            \
                      static_cast<const Elem<TT>::S*>(v), v_stride, workspace, state, cu_seqlens, positions,          \
@@ -1058,11 +1111,17 @@ extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_s
                        r_stride, static_cast<const E*>(k), k_stride, static_cast<const E*>(decay), decay_stride,
                        decay_bias, static_cast<const E*>(rate), rate_stride, rate_bias, num_heads, head_dim,
                        static_cast<int>(dp));
-    if (dp == 32) MI355_GDELTA(TT, 8, 4, 4);
+    if (!long_chunks) {
+      if (dp == 32) MI355_GCOLS(32);
+      else if (dp == 64) MI355_GCOLS(64);
+      else if (dp == 128) MI355_GCOLS(128);
+      else MI355_GCOLS(256);
+    } else if (dp == 32) MI355_GDELTA(TT, 8, 4, 4);
     else if (dp == 64) MI355_GDELTA(TT, 16, 4, 4);
     else if (dp == 128) MI355_GDELTA(TT, 16, 8, 2);
     else MI355_GDELTA(TT, 16, 16, 1);
   });
 #undef MI355_GDELTA
+#undef MI355_GCOLS
   return check_launch("general_delta_rule");
 }

@@ -114,7 +114,7 @@ def _load() -> ctypes.CDLL:
         "mi355_gated_delta_rule_workspace": (I64, [I64, I32, I32, I32]),
         "mi355_general_delta_rule_workspace": (I64, [I64, I32, I32]),
         "mi355_general_delta_rule": (I32, [P, P, I64, P, I64, P, I64, P, I64, P, P, I64, P, P, P, P, P, I32, I32, I32, I64,
-                                           P, I64, I32, P]),
+                                           I32, P, I64, I32, P]),
         "mi355_group_rms_norm_f32": (I32, [P, P, P, P, I64, I32, I32, F, I32, P]),
         "mi355_gated_norm_resid_f32": (I32, [P, P, P, I64, P, P, I64, I32, I32, F, F, I32, P]),
         "mi355_rms_norm_rows": (I32, [P, P, I64, P, I64, I32, F, I32, P]),

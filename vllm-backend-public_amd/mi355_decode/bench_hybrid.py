@@ -20,7 +20,31 @@ from .config import EngineArgs, ModelConfig
 HBM, MFMA, VALU = 8.0e12, 2.5e15, 157.3e12
 
 
-def lozupel_config(width: int, layers: int, vocab: int = 32000) -> dict:
+def tativik_config(width: int, layers: int, vocab: int = 32000) -> dict:
+    """Alternating general-delta / latent-attention layers (every second attention reads the latent
+    pages of the one before it), 64-wide recurrent heads, 128 + 64-wide attention heads over a latent of
+    512, a 1024-token window, and in every layer 32 experts of width / 2 of which 4 run per token:
+    as many active feed-forward weights as a dense feed-forward of 2 * width."""
+    nh = width // 128
+    ls, last_latent = [], None
+    moe = {"kind": "moe", "expert": {"ff": width // 2},
+           "router": {"experts": 32, "top": 4, "groups": {"count": 4, "keep": 2}}}
+    for i in range(layers):
+        if i % 2 == 0:
+            ls.append({"type": "general_delta", "mixer": {"heads": width // 64, "dim": 64}, "mlp": moe})
+            continue
+        m = {"heads": nh, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": max(width * 3 // 8, 256),
+             "mask": {"size": 1024}, "rot": {"dims": 64, "base": 1.0e6}, "scale": 192 ** -0.5}
+        if last_latent is not None:
+            m["kv_from"], last_latent = last_latent, None
+        else:
+            last_latent = i
+        ls.append({"type": "latent_attention", "mixer": m, "mlp": moe})
+    return {"architecture": "Tativik", "width": width, "vocab": vocab, "norm": {"eps": 1e-6, "groups": 4},
+            "residual_mult": 0.7, "layers": ls}
+
+
+def lozupel_config(width: int, layers: int, vocab: int = 32000, loop: bool = True) -> dict:
     """Alternating parallel / delta layers with 128-wide heads, a 1024-token window, a feed-forward in
     every layer; the middle of the stack loops twice."""
     nh = width // 128
@@ -33,7 +57,7 @@ def lozupel_config(width: int, layers: int, vocab: int = 32000) -> dict:
            {"type": "delta", "mixer": delta, "mlp": ff}) for i in range(layers)]
     d = {"architecture": "Lozupel", "embedding": {"scale": 1.0}, "width": width, "vocab": vocab, "norm": {"eps": 1e-6},
          "logit_softcap": 30.0, "layers": ls}
-    if layers >= 3:
+    if layers >= 3 and loop:
         d["loop"] = {"start": 1, "stop": layers - 1, "times": 2}
     return d
 
@@ -226,4 +250,151 @@ def compare(widths, layers: int, batch: int, prompt_len: int, steps: int, warmup
                                  "prefill_ratio": round(h["prefill_tok_s"] / ll["prefill_tok_s"], 3),
                                  "decode_ratio": round(h["decode_tok_s"] / ll["decode_tok_s"], 3)})
         result["kernels"][str(width)] = kernel_table(width, prompt_len, batch)
+    return result
+
+
+def tativik_kernel_table(width: int, prompt_len: int, batch: int) -> list:
+    """The sandwich arrangement's kernels at the prefill and the decode shape, each against its own
+    roofline, beside the like kernel of the "pre" arrangement (the Lozupel design) at the same shape."""
+    from types import SimpleNamespace
+    from .config import MoESpec
+    from .hybrid_runner import MoEFeedForward, rotary_table
+    dev, bf = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rnd = lambda *s, dt=bf: torch.randn(*s, device=dev, dtype=torch.float32, generator=g).to(dt)  # noqa: E731
+    rows = []
+
+    def row(kernel, shape, t, bound, work, like=None, like_t=None, like_work=None, like_bound=None):
+        peak = {"hbm": HBM, "mfma": MFMA, "valu": VALU}
+        r = {"kernel": kernel, "shape": shape, "us": round(t * 1e6, 2), "bound": bound,
+             "frac_of_roofline": round(work / peak[bound] / t, 4)}
+        if like is not None:
+            r.update(like=like, like_us=round(like_t * 1e6, 2), like_frac=round(like_work / peak[like_bound or bound] / like_t, 4))
+            r["distance_ratio"] = round(r["like_frac"] / max(r["frac_of_roofline"], 1e-9), 2)
+        rows.append(r)
+
+    P, W = prompt_len, width
+    for T, tag in ((P, "prefill"), (batch, "decode")):
+        shape = f"{tag} {T} rows x {W}"
+        resid, add16, w1 = rnd(T, W, dt=torch.float32), rnd(T, W), rnd(1)
+        wv32, b32, out16 = rnd(W, dt=torch.float32), rnd(W, dt=torch.float32), torch.empty(T, W, device=dev, dtype=bf)
+        row("group_rms_norm_f32 (4 groups)", shape, _time(lambda: ops.group_rms_norm_f32(resid, wv32, 4, 1e-6, dtype=bf, out=out16)),
+            "hbm", T * W * 6, "add_rms_norm_f32", _time(lambda: ops.add_rms_norm_f32(resid, w1, 1e-6, out=out16)), T * W * 6)
+        y, gate, wv = rnd(T, W), rnd(T, W), rnd(W)
+        row("gated_norm_resid_f32 (4 groups)", shape,
+            _time(lambda: ops.gated_norm_resid_f32(resid, y, gate, b32, wv32, 4, 1e-6, 0.7)), "hbm", T * W * 12,
+            "rms_norm_mix_f32 (two inputs)", _time(lambda: ops.rms_norm_mix_f32(resid, y, wv, gate, wv, 1e-6, 0.5)), T * W * 12)
+
+    # ---- attention: one prompt of P tokens; then `batch` sequences decoding at that context
+    H, R_, rot, window = W // 128, 512, 64, 1024
+    G, d, dv = max(W // 512, 1), 128, 128
+    pages = (P + BLOCK_SIZE) // BLOCK_SIZE + 1
+    nb = pages * batch
+    cache = rnd(nb, BLOCK_SIZE, R_ + rot)
+    kc, vct = rnd(nb, G, BLOCK_SIZE, d), rnd(nb, G, dv, BLOCK_SIZE)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev).view(batch, pages)
+    cs = rotary_table(rot, 1.0e6, pages * BLOCK_SIZE, dev)
+    sink, temp, bias = torch.zeros(H, device=dev), torch.ones(H, device=dev), torch.full((H,), -2.0, device=dev)
+    keys = sum(min(i + 1, window) for i in range(P))
+    for T, tag in ((P, "prefill"), (batch, "decode")):
+        ql, q, gt = rnd(H, T, R_) * 0.05, rnd(T, H * (128 + rot)), rnd(T, H)
+        qs = rnd(T, H * d)
+        if tag == "prefill":
+            pos, seq, b_t = torch.arange(P, dtype=torch.int64, device=dev), torch.zeros(P, dtype=torch.int32, device=dev), bt[:1]
+            tiles = torch.from_numpy(ops.query_tiles([0, P])).to(dev)
+            nsp = max(min(16, 2048 // max(tiles.shape[0] * G * max(H // G // 4, 1), 1)), 1)
+            nkeys, shape = keys, f"prefill {P} tokens, window {window}"
+        else:
+            pos, seq, b_t = torch.full((T,), P - 1, dtype=torch.int64, device=dev), torch.arange(T, dtype=torch.int32, device=dev), bt
+            tiles = torch.stack([seq, seq, torch.ones_like(seq)], dim=1).contiguous()
+            nsp, nkeys, shape = 16, T * min(P, window), f"decode {T} rows at context {P}, window {window}"
+        part = torch.empty(nsp * T * H * dv, device=dev)
+        ol, o = torch.empty(H, T, R_, device=dev, dtype=bf), torch.empty(T, H * dv, device=dev, dtype=bf)
+        t_n = _time(lambda: ops.latent_window_attn(ql, q, 128 + rot, 128, cache, b_t, seq, pos, sink, gt, cs, window, 0.07,
+                                                   out=ol, **latent_attn_extra(T, tiles)), 5)
+        t_l = _time(lambda: ops.sigmoid_window_attn(qs, kc, vct, b_t, seq, pos, temp, bias, gt, H, window, d ** -0.5, out=o,
+                                                    tiles=tiles, partial=part, num_splits=nsp), 5)
+        if tag == "prefill":
+            row("latent_window_attn", f"{shape}, {H} heads x ({R_} + {rot})", t_n, "mfma", 2.0 * nkeys * H * (2 * R_ + rot),
+                f"sigmoid_window_attn, {H}/{G} heads x {d}", t_l, 2.0 * nkeys * H * (d + dv))
+        else:
+            row("latent_window_attn", f"{shape}, {H} heads x ({R_} + {rot})", t_n, "hbm", nkeys * (R_ + rot) * 2,
+                f"sigmoid_window_attn, {H}/{G} heads x {d}", t_l, nkeys * G * (d + dv) * 2)
+        x, nw = rnd(T, R_ + rot), torch.ones(R_, device=dev)
+        slots = (torch.arange(T, device=dev) if tag == "prefill" else torch.arange(T, device=dev) * pages * BLOCK_SIZE + P - 1).to(torch.int64)
+        k_, v_ = rnd(T, G * d), rnd(T, G * dv)
+        cs2 = rotary_table(64, 1.0e6, pages * BLOCK_SIZE, dev)
+        row("latent_kv_write (norm + rotation)", f"{tag} {T} rows x {R_ + rot}",
+            _time(lambda: ops.latent_kv_write(x, nw, cs, pos, slots, cache, R_, rot, 1e-6)), "hbm", T * (R_ + rot) * 4,
+            "rope_partial_kv_write", _time(lambda: ops.rope_partial_kv_write(qs, k_, v_, cs2, pos, slots, kc, vct, H, G, d, dv)),
+            T * (2 * H * d + 2 * G * (d + dv)) * 2)
+
+    # ---- the recurrences: heads of 64 x 64 state beside the gated rule's 128 x 128, equal state per layer
+    Hn, dn = W // 64, 64
+    Hd, Gd, dd = W // 128, max(W // 256, 1), 128
+    for T, S, tag in ((P, 1, "prefill"), (batch, batch, "decode")):
+        per = T // S
+        cu_ = torch.arange(0, T + 1, per, dtype=torch.int32, device=dev)
+        pos_ = (torch.arange(T, device=dev) % per + (0 if S == 1 else P)).to(torch.int64)
+        slots = torch.arange(S, dtype=torch.int32, device=dev)
+        xn = rnd(T, 5 * Hn * dn)
+        C = Hn * dn
+        w0, ab = torch.zeros(C, device=dev), torch.zeros(C, device=dev)
+        stn = torch.zeros(S + 1, Hn, dn, dn, device=dev)
+        on = torch.empty(T, Hn, dn, device=dev)
+        t_n = _time(lambda: ops.general_delta_rule(xn[:, :C], xn[:, C:2 * C], xn[:, 2 * C:3 * C], xn[:, 3 * C:4 * C], w0,
+                                                   xn[:, 4 * C:], ab, stn, cu_, pos_, slots, Hn, dn, out=on, long_chunks=S == 1), 5)
+        Cd = 2 * Gd * dd + Hd * dd
+        xd, beta, dec = rnd(T, Cd), rnd(T, Hd), rnd(T, Hd)
+        a_log, dtb = torch.zeros(Hd, device=dev), torch.zeros(Hd, device=dev)
+        std = torch.zeros(S + 1, Hd, dd, dd, device=dev)
+        od = torch.empty(T, Hd, dd, device=dev)
+        t_l = _time(lambda: ops.gated_delta_rule(xd, 0, Gd * dd, 2 * Gd * dd, beta, dec, a_log, dtb, std, cu_, pos_, slots, Hd,
+                                                 Gd, dd, dd, out=od, long_chunks=S == 1), 5)
+        if S == 1:
+            row("general_delta_rule", f"prefill {T} tokens, {Hn} heads x {dn} x {dn}", t_n, "valu", 8.0 * T * Hn * dn * dn,
+                f"gated_delta_rule, {Hd} heads x {dd} x {dd}", t_l, 6.0 * T * Hd * dd * dd)
+        else:
+            row("general_delta_rule", f"decode {S} rows, {Hn} heads x {dn} x {dn}", t_n, "hbm", S * Hn * dn * dn * 8,
+                f"gated_delta_rule, {Hd} heads x {dd} x {dd}", t_l, S * Hd * dd * dd * 8)
+
+    # ---- the mixture of experts beside a dense gated feed-forward with as many active weights
+    E, top, F = 32, 4, W // 2
+    lw = SimpleNamespace(router_w=rnd(E, W, dt=torch.float32) * W ** -0.5, correction=torch.zeros(E, device=dev),
+                         gate_up_w=rnd(E, 2 * F, W) * W ** -0.5, down_w=rnd(E, W, F) * F ** -0.5)
+    ff = MoEFeedForward(MoESpec(E, top, 4, 2, F), lw, None)
+    gu_w, dn_w = rnd(2 * top * F, W) * W ** -0.5, rnd(W, top * F) * F ** -0.5
+    for T, tag in ((P, "prefill"), (batch, "decode")):
+        h = rnd(T, W)
+        t_n = _time(lambda: ff(h), 5)
+        if tag == "prefill":
+            dense = lambda: torch.mm(ops.gelu_tanh_and_mul(torch.mm(h, gu_w.t())), dn_w.t())   # noqa: E731
+            row("mixture of experts (route, sort, expert GEMMs, sum)", f"prefill {T} rows, {top} of {E} experts x {F}", t_n,
+                "mfma", 6.0 * T * top * F * W, "dense gated feed-forward (library GEMMs)", _time(dense, 5), 6.0 * T * top * F * W)
+        else:
+            dense = lambda: ops.linear_decode(ops.gelu_tanh_and_mul(ops.linear_decode(h, gu_w)), dn_w)   # noqa: E731
+            touched = min(E, T * top)
+            row("mixture of experts (route, sort, per-row products, sum)", f"decode {T} rows, {top} of {E} experts x {F}", t_n,
+                "hbm", touched * 3 * F * W * 2, "dense gated feed-forward (weight stream)", _time(dense, 5), 3 * top * F * W * 2)
+    return rows
+
+
+def latent_attn_extra(T: int, tiles) -> dict:
+    """Keyword arguments that select the latent attention's form for a step of T rows."""
+    return {}
+
+
+def compare_tativik(widths, layers: int, batch: int, prompt_len: int, steps: int, warmup: int) -> dict:
+    """The sandwich arrangement (Tativik) beside the closest existing model, the "pre" arrangement
+    (Lozupel), at equal width and depth and as many active feed-forward weights."""
+    result = {"metric": "tativik_vs_lozupel_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+              "config": {"layers": layers, "batch": batch, "prompt_len": prompt_len, "decode_steps": steps},
+              "models": [], "kernels": {}}
+    for width in widths:
+        t = through_engine(ModelConfig.from_dict(tativik_config(width, layers)), batch, prompt_len, steps, warmup)
+        z = through_engine(ModelConfig.from_dict(lozupel_config(width, layers, loop=False)), batch, prompt_len, steps, warmup)
+        result["models"].append({"width": width, "layers": layers, "tativik": t, "lozupel": z,
+                                 "prefill_ratio": round(t["prefill_tok_s"] / z["prefill_tok_s"], 3),
+                                 "decode_ratio": round(t["decode_tok_s"] / z["decode_tok_s"], 3)})
+        result["kernels"][str(width)] = tativik_kernel_table(width, prompt_len, batch)
     return result

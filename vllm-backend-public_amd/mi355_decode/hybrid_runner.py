@@ -121,7 +121,7 @@ class GeneralDeltaMixer:
         col = lambda n: proj[:, lw.seg[n][0]: lw.seg[n][0] + lw.seg[n][1]]     # noqa: E731
         decay = r.linear(ops.tanh_rows(col("w1")), lw.w2_w)
         o = ops.general_delta_rule(col("r"), col("k"), col("v"), decay, lw.w0, col("a"), lw.a_b, r.rec_state[self.si],
-                                   b.cu_seqlens, b.positions, b.state_slots, s.heads, s.dim)
+                                   b.cu_seqlens, b.positions, b.state_slots, s.heads, s.dim, long_chunks=b.long_chunks)
         return r.linear(ops.gated_head_rms_norm(o, col("g"), lw.head_norm, r.eps, ops.ACT_SIGMOID), lw.o_w)
 
 
@@ -164,17 +164,31 @@ class MoEFeedForward:
         offsets, perm, inv = ops.moe_sort(ids, s.experts)
         rows = T * s.top
         if rows >= self.GROUPED_MIN_ROWS and not torch.cuda.is_current_stream_capturing():
-            xs = ops.moe_gather_rows(h, perm, rows, s.top)
-            off = offsets.tolist()
-            gu = torch.empty(rows, 2 * s.ff, dtype=h.dtype, device=h.device)
-            for e in range(s.experts):
-                if off[e + 1] > off[e]:
-                    torch.mm(xs[off[e]: off[e + 1]], lw.gate_up_w[e].t(), out=gu[off[e]: off[e + 1]])
-            act = ops.moe_silu_and_mul(gu)
-            y = torch.empty(rows, h.shape[1], dtype=h.dtype, device=h.device)
-            for e in range(s.experts):
-                if off[e + 1] > off[e]:
-                    torch.mm(act[off[e]: off[e + 1]], lw.down_w[e].t(), out=y[off[e]: off[e + 1]])
+            # many rows: library GEMMs per expert.  The largest count comes to the host (one wait); when the
+            # experts' loads are near even, every expert's rows are padded to that count and the two products
+            # are one batched GEMM each; otherwise one GEMM per expert on its range of the sorted rows.
+            counts = offsets[1:] - offsets[:-1]
+            cap = -(-int(counts.max()) // 16) * 16
+            if s.experts * cap <= 2 * rows:
+                at = offsets[:-1].long()[:, None] + torch.arange(cap, device=h.device)[None, :]
+                tok = perm.long()[at.clamp_(max=rows - 1).view(-1)] // s.top      # past an expert's count: some row, unused
+                gu = torch.bmm(h.index_select(0, tok).view(s.experts, cap, -1), lw.gate_up_w.transpose(1, 2))
+                act = ops.moe_silu_and_mul(gu.view(s.experts * cap, 2 * s.ff))
+                y = torch.bmm(act.view(s.experts, cap, s.ff), lw.down_w.transpose(1, 2)).view(s.experts * cap, -1)
+                e = ids.view(-1).long()
+                inv = (inv[:rows].long() + e * cap - offsets.long()[e]).to(torch.int32)
+            else:
+                xs = ops.moe_gather_rows(h, perm, rows, s.top)
+                off = offsets.tolist()
+                gu = torch.empty(rows, 2 * s.ff, dtype=h.dtype, device=h.device)
+                for e in range(s.experts):
+                    if off[e + 1] > off[e]:
+                        torch.mm(xs[off[e]: off[e + 1]], lw.gate_up_w[e].t(), out=gu[off[e]: off[e + 1]])
+                act = ops.moe_silu_and_mul(gu)
+                y = torch.empty(rows, h.shape[1], dtype=h.dtype, device=h.device)
+                for e in range(s.experts):
+                    if off[e + 1] > off[e]:
+                        torch.mm(act[off[e]: off[e + 1]], lw.down_w[e].t(), out=y[off[e]: off[e + 1]])
         else:
             y = ops.moe_down_rows(ops.moe_gate_up_rows(h, lw.gate_up_w, offsets, perm, s.top), lw.down_w, offsets)
         return ops.moe_combine(y, inv, wts, T, s.top)

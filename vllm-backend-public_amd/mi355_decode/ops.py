@@ -1196,11 +1196,12 @@ def gated_delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, beta
 def general_delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, decay_bias: torch.Tensor,
                        rate: torch.Tensor, rate_bias: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
                        positions: torch.Tensor, state_slots: torch.Tensor, num_heads: int, head_dim: int,
-                       out: torch.Tensor | None = None):
+                       out: torch.Tensor | None = None, long_chunks: bool = True):
     """The general delta rule over packed chunks: S <- diag(w) S - (a u)(u^T S) + k v^T, o = S^T r with
     w = exp(-exp(-1/2) sigmoid(decay + decay_bias)), a = sigmoid(rate + rate_bias), u the unit key.
     r / k / v / decay / rate [tokens, heads * head_dim] (column slices are fine); the biases float32;
-    state float32 [slots, heads, head_dim, head_dim].  Returns o float32 [tokens, heads, head_dim]."""
+    state float32 [slots, heads, head_dim, head_dim].  Returns o float32 [tokens, heads, head_dim].
+    long_chunks False: the form for chunks of a token or two (one state column per lane)."""
     dt = _dt3(r, "r")
     T, C = r.shape[0], num_heads * head_dim
     S = cu_seqlens.numel() - 1
@@ -1216,8 +1217,8 @@ def general_delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay:
         _cols(v, "v", C), _same(decay, r, "decay"), _cols(decay, "decay", C), _f32(decay_bias, "decay_bias", C),
         _same(rate, r, "rate"), _cols(rate, "rate", C), _f32(rate_bias, "rate_bias", C), _f32(state, "state"),
         _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(positions, "positions", torch.int64, T),
-        _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, head_dim, T, ws.data_ptr(), ws.numel(), dt,
-        _stream()))
+        _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, head_dim, T, int(bool(long_chunks)), ws.data_ptr(),
+        ws.numel(), dt, _stream()))
     return out
 
 
