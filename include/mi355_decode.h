@@ -889,7 +889,8 @@ int32_t mi355_tanh_rows(void* out, const void* x, int64_t x_stride, int64_t num_
  *   latent_kv_write      x [tokens, rank + rot] (a column slice is fine): c = x[:rank] / rms * norm_weight,
  *                        the last rot columns rotated (first rot_dims of them, coordinate i with
  *                        i + rot_dims / 2, table cos_sin [max_pos, rot_dims] = cos | sin), into the
- *                        row's page slot; rows with slot < 0 store nothing
+ *                        row's page slot; rows with slot < 0 store nothing.  cache_t (may be null):
+ *                        a second, channel-major copy of the latent, [blocks, rank, 16]
  *   latent_window_attn   out[t, h] = sigmoid(gate[t, h]) * sum_j p_j c_j over the keys j of the row's
  *                        sequence with 0 <= p - j < window,
  *                        p_j = exp(s_j) / (exp(sink[h]) + sum_j' exp(s_j')),
@@ -900,10 +901,36 @@ int32_t mi355_tanh_rows(void* out, const void* x, int64_t x_stride, int64_t num_
  *                        rotate at q_rot_offset of every head.  out: rank numbers per (t, h), strides
  *                        likewise; the caller applies the value up-projection.  gate may be null.
  */
-int32_t mi355_latent_kv_write(void* cache, const void* x, int64_t x_stride, const float* norm_weight,
+int32_t mi355_latent_kv_write(void* cache, void* cache_t, const void* x, int64_t x_stride,
+                              const float* norm_weight,
                               const float* cos_sin, int32_t max_pos, const int64_t* positions,
                               const int64_t* slot_mapping, int64_t num_tokens, int32_t rank,
                               int32_t rot, int32_t rot_dims, float eps, int32_t dtype, void* stream);
+/*
+ * The matrix-core form of latent_window_attn (16-bit storage, rank a multiple of 16 up to 512,
+ * rank + rot a multiple of 8 up to 640), same result.
+ *   latent_q_pack              q_packed [tokens, heads, rank + rot] = q_latent | rotated part of q
+ *   latent_window_attn_tiles   tiles [num_tiles][3] = (chunk, first pair, pairs <= 16): a pair is
+ *                              (packed row, head), number row * heads + head; a tile's pairs are
+ *                              consecutive and of one chunk, every pair in exactly one tile.  Reads both
+ *                              copies of the latent (see latent_kv_write).  num_splits > 1: the keys
+ *                              of a tile are dealt out to that many workgroups and merged by a second
+ *                              launch; partial: num_splits * tokens * heads * (rank + 2) floats
+ */
+int32_t mi355_latent_q_pack(void* q_packed, const void* q_latent, int64_t q_latent_stride,
+                            int64_t q_latent_head_stride, const void* q, int64_t q_stride,
+                            int32_t q_head_width, int32_t q_rot_offset, const float* cos_sin,
+                            int32_t max_pos, const int64_t* positions, int64_t num_tokens,
+                            int32_t num_heads, int32_t rank, int32_t rot, int32_t rot_dims,
+                            int32_t dtype, void* stream);
+int32_t mi355_latent_window_attn_tiles(void* out, int64_t out_stride, int64_t out_head_stride,
+                                       const void* q_packed, const void* cache, const void* cache_t,
+                                       const int32_t* block_tables, int32_t max_blocks,
+                                       const int32_t* tiles, int32_t num_tiles,
+                                       const int64_t* positions, const float* sink, const void* gate,
+                                       int64_t gate_stride, int64_t num_tokens, int32_t num_heads,
+                                       int32_t rank, int32_t rot, int32_t window, float scale,
+                                       float* partial, int32_t num_splits, int32_t dtype, void* stream);
 int32_t mi355_latent_window_attn(void* out, int64_t out_stride, int64_t out_head_stride,
                                  const void* q_latent, int64_t q_latent_stride,
                                  int64_t q_latent_head_stride, const void* q, int64_t q_stride,

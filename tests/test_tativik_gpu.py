@@ -252,7 +252,8 @@ def _paged(T, num_pages, seed):
     return order, order[pos // 16].astype(np.int64) * 16 + pos % 16
 
 
-def _latent_in_cuts(x, nw, ql, q, hw, off, sink, gate, cuts, H, R_, rot, dims, window, scale, base=100.0, pages=12):
+def _latent_in_cuts(x, nw, ql, q, hw, off, sink, gate, cuts, H, R_, rot, dims, window, scale, base=100.0, pages=12,
+                    tiled=False):
     """Latent write + attention over one sequence fed in portions (a last portion takes what `cuts`
     leaves); returns [T, H, R_] float32."""
     from mi355_decode import ops
@@ -261,6 +262,7 @@ def _latent_in_cuts(x, nw, ql, q, hw, off, sink, gate, cuts, H, R_, rot, dims, w
     cuts = list(cuts) + [T]
     table, slots = _paged(T, pages, 5)
     cache = torch.full((pages, 16, R_ + rot), float("nan"), dtype=dt, device="cuda")
+    cache_t = torch.full((pages, R_, 16), float("nan"), dtype=dt, device="cuda") if tiled else None
     bt = torch.zeros(1, pages, dtype=torch.int32)
     bt[0, : len(table)] = torch.from_numpy(table)
     cs = rotary_table(dims, base, pages * 16, "cuda")
@@ -271,10 +273,18 @@ def _latent_in_cuts(x, nw, ql, q, hw, off, sink, gate, cuts, H, R_, rot, dims, w
             break
         sl = slice(at, at + n)
         pos = torch.arange(at, at + n, dtype=torch.int64, device="cuda")
-        ops.latent_kv_write(x[sl].cuda(), nw.cuda(), cs, pos, torch.from_numpy(slots[sl]).cuda(), cache, R_, rot, 1e-5)
-        out = ops.latent_window_attn(ql[sl].transpose(0, 1).contiguous().cuda(), q[sl].cuda(), hw, off, cache, bt.cuda(),
-                                     torch.zeros(n, dtype=torch.int32, device="cuda"), pos, sink.cuda(),
-                                     None if gate is None else gate[sl].cuda(), cs, window, scale)
+        ops.latent_kv_write(x[sl].cuda(), nw.cuda(), cs, pos, torch.from_numpy(slots[sl]).cuda(), cache, R_, rot, 1e-5,
+                            cache_t=cache_t)
+        qlh = ql[sl].transpose(0, 1).contiguous().cuda()
+        if tiled:                                             # the matrix cores; single rows spread their keys over three workgroups
+            out = ops.latent_window_attn_tiles(ops.latent_q_pack(qlh, q[sl].cuda(), hw, off, rot, cs, pos), cache, cache_t,
+                                               bt.cuda(), torch.from_numpy(ops.pair_tiles([0, n], H)).cuda(), pos, sink.cuda(),
+                                               None if gate is None else gate[sl].cuda(), window, scale,
+                                               num_splits=3 if n == 1 else 1)
+        else:
+            out = ops.latent_window_attn(qlh, q[sl].cuda(), hw, off, cache, bt.cuda(),
+                                         torch.zeros(n, dtype=torch.int32, device="cuda"), pos, sink.cuda(),
+                                         None if gate is None else gate[sl].cuda(), cs, window, scale)
         outs.append(out.float().cpu().transpose(0, 1))
         at += n
     assert at == T
@@ -317,6 +327,25 @@ def test_latent_attention_whole_portions_and_single_tokens(H, R_, rot, dims, win
     assert (got - ref).abs().max() <= 3e-2 * ref.abs().max()
 
 
+@pytest.mark.parametrize("H,R_,rot,dims,window", [(3, 48, 8, 4, 20), (2, 64, 16, 16, 1), (4, 96, 32, 32, 33), (1, 128, 8, 0, 200),
+                                                  (16, 128, 64, 64, 48), (20, 512, 64, 32, 17), (5, 208, 24, 24, 40)])
+def test_latent_attention_on_the_matrix_cores(H, R_, rot, dims, window):
+    """bfloat16 inputs; the restatement sees the same rounded inputs, so what is left is the rounding of
+    the stored latent, of the packed query and of the weights in the second product."""
+    g = torch.Generator().manual_seed(H * 100 + R_)
+    T, hw, off = 75, rot + 8, 8
+    b16 = lambda t: t.to(torch.bfloat16)                      # noqa: E731
+    x = b16(torch.randn(T, R_ + rot, generator=g))
+    nw, sink = torch.randn(R_, generator=g) * 0.2 + 1, torch.randn(H, generator=g)
+    ql, q = b16(torch.randn(T, H, R_, generator=g) * 0.5), b16(torch.randn(T, H * hw, generator=g))
+    gate = b16(torch.randn(T, H, generator=g))
+    args = (H, R_, rot, dims, window, 0.3)
+    ref = _latent_ref(x, nw, ql, q, hw, off, sink, gate, *args)
+    for cuts in ([T], [1] * T, [2, 3, 1, 30, 2, 16, 21]):
+        got = _latent_in_cuts(x, nw, ql, q, hw, off, sink, gate, cuts, *args, tiled=True)
+        assert (got - ref).abs().max() <= 3e-2 * ref.abs().max(), cuts
+
+
 @pytest.mark.parametrize("window", [16, 17, 31, 48, 64, 65])
 def test_latent_window_edge_and_sink_show_with_one_loud_key(window):
     """Token 9 holds a latent that every query scores far above all others: a query sees it exactly
@@ -339,6 +368,10 @@ def test_latent_window_edge_and_sink_show_with_one_loud_key(window):
     for cuts in ([T], [9 + window - 1, 1, 1] + [1] * 5, [5, 2] + [1] * (T - 7)):
         got = _latent_in_cuts(x, nw, ql, q, rot, 0, sink, None, cuts, *args)
         assert (got - ref).abs().max() <= 1e-4 * ref.abs().max(), cuts
+        b16 = lambda t: t.to(torch.bfloat16)                  # noqa: E731
+        got = _latent_in_cuts(b16(x), nw, b16(ql), b16(q), rot, 0, sink, None, cuts, *args, tiled=True)
+        r16 = _latent_ref(b16(x), nw, b16(ql), b16(q), rot, 0, sink, None, *args)
+        assert (got - r16).abs().max() <= 3e-2 * r16.abs().max(), cuts
 
 
 def test_routing_groups_corrections_and_negative_choice_scores():

@@ -119,7 +119,10 @@ def _load() -> ctypes.CDLL:
         "mi355_gated_norm_resid_f32": (I32, [P, P, P, I64, P, P, I64, I32, I32, F, F, I32, P]),
         "mi355_rms_norm_rows": (I32, [P, P, I64, P, I64, I32, F, I32, P]),
         "mi355_tanh_rows": (I32, [P, P, I64, I64, I32, I32, P]),
-        "mi355_latent_kv_write": (I32, [P, P, I64, P, P, I32, P, P, I64, I32, I32, I32, F, I32, P]),
+        "mi355_latent_kv_write": (I32, [P, P, P, I64, P, P, I32, P, P, I64, I32, I32, I32, F, I32, P]),
+        "mi355_latent_q_pack": (I32, [P, P, I64, I64, P, I64, I32, I32, P, I32, P, I64, I32, I32, I32, I32, I32, P]),
+        "mi355_latent_window_attn_tiles": (I32, [P, I64, I64, P, P, P, P, I32, P, I32, P, P, P, I64, I64, I32, I32, I32, I32,
+                                                 F, P, I32, I32, P]),
         "mi355_latent_window_attn": (I32, [P, I64, I64, P, I64, I64, P, I64, I32, I32, P, P, I32, P, P, P, P, I64, P, I32,
                                            I64, I32, I32, I32, I32, I32, F, I32, P]),
         "mi355_moe_route": (I32, [P, P, P, P, I64, I32, I32, I32, I32, P]),
@@ -165,6 +168,7 @@ EXPORTS = ("mi355_abi_version", "mi355_last_error", "mi355_target_arch",
            "mi355_conv_state_update", "mi355_gated_delta_rule", "mi355_gated_delta_rule_workspace",
            "mi355_general_delta_rule", "mi355_general_delta_rule_workspace", "mi355_group_rms_norm_f32",
            "mi355_gated_norm_resid_f32", "mi355_rms_norm_rows", "mi355_tanh_rows", "mi355_latent_kv_write",
+           "mi355_latent_q_pack", "mi355_latent_window_attn_tiles",
            "mi355_latent_window_attn", "mi355_moe_route", "mi355_moe_sort", "mi355_moe_gather_rows",
            "mi355_moe_gate_up_rows", "mi355_moe_down_rows", "mi355_moe_silu_and_mul", "mi355_moe_combine")
 

@@ -290,7 +290,7 @@ def tativik_kernel_table(width: int, prompt_len: int, batch: int) -> list:
     G, d, dv = max(W // 512, 1), 128, 128
     pages = (P + BLOCK_SIZE) // BLOCK_SIZE + 1
     nb = pages * batch
-    cache = rnd(nb, BLOCK_SIZE, R_ + rot)
+    cache, cache_t = rnd(nb, BLOCK_SIZE, R_ + rot), rnd(nb, R_, BLOCK_SIZE)
     kc, vct = rnd(nb, G, BLOCK_SIZE, d), rnd(nb, G, dv, BLOCK_SIZE)
     bt = torch.arange(nb, dtype=torch.int32, device=dev).view(batch, pages)
     cs = rotary_table(rot, 1.0e6, pages * BLOCK_SIZE, dev)
@@ -310,8 +310,12 @@ def tativik_kernel_table(width: int, prompt_len: int, batch: int) -> list:
             nsp, nkeys, shape = 16, T * min(P, window), f"decode {T} rows at context {P}, window {window}"
         part = torch.empty(nsp * T * H * dv, device=dev)
         ol, o = torch.empty(H, T, R_, device=dev, dtype=bf), torch.empty(T, H * dv, device=dev, dtype=bf)
-        t_n = _time(lambda: ops.latent_window_attn(ql, q, 128 + rot, 128, cache, b_t, seq, pos, sink, gt, cs, window, 0.07,
-                                                   out=ol, **latent_attn_extra(T, tiles)), 5)
+        cu_h = [0, P] if tag == "prefill" else list(range(T + 1))
+        ptiles = torch.from_numpy(ops.pair_tiles(cu_h, H)).to(dev)
+        qe = ops.latent_q_pack(ql, q, 128 + rot, 128, rot, cs, pos)
+        nspl = min(16, max(window // 64, 1), max(1024 // int(ptiles.shape[0]), 1))
+        t_n = _time(lambda: ops.latent_window_attn_tiles(qe, cache, cache_t, b_t, ptiles, pos, sink, gt, window, 0.07,
+                                                         num_splits=nspl, out=ol), 5)
         t_l = _time(lambda: ops.sigmoid_window_attn(qs, kc, vct, b_t, seq, pos, temp, bias, gt, H, window, d ** -0.5, out=o,
                                                     tiles=tiles, partial=part, num_splits=nsp), 5)
         if tag == "prefill":
@@ -325,7 +329,8 @@ def tativik_kernel_table(width: int, prompt_len: int, batch: int) -> list:
         k_, v_ = rnd(T, G * d), rnd(T, G * dv)
         cs2 = rotary_table(64, 1.0e6, pages * BLOCK_SIZE, dev)
         row("latent_kv_write (norm + rotation)", f"{tag} {T} rows x {R_ + rot}",
-            _time(lambda: ops.latent_kv_write(x, nw, cs, pos, slots, cache, R_, rot, 1e-6)), "hbm", T * (R_ + rot) * 4,
+            _time(lambda: ops.latent_kv_write(x, nw, cs, pos, slots, cache, R_, rot, 1e-6, cache_t=cache_t)), "hbm",
+            T * (3 * R_ + 2 * rot) * 2,
             "rope_partial_kv_write", _time(lambda: ops.rope_partial_kv_write(qs, k_, v_, cs2, pos, slots, kc, vct, H, G, d, dv)),
             T * (2 * H * d + 2 * G * (d + dv)) * 2)
 
@@ -377,11 +382,6 @@ def tativik_kernel_table(width: int, prompt_len: int, batch: int) -> list:
             row("mixture of experts (route, sort, per-row products, sum)", f"decode {T} rows, {top} of {E} experts x {F}", t_n,
                 "hbm", touched * 3 * F * W * 2, "dense gated feed-forward (weight stream)", _time(dense, 5), 3 * top * F * W * 2)
     return rows
-
-
-def latent_attn_extra(T: int, tiles) -> dict:
-    """Keyword arguments that select the latent attention's form for a step of T rows."""
-    return {}
 
 
 def compare_tativik(widths, layers: int, batch: int, prompt_len: int, steps: int, warmup: int) -> dict:

@@ -48,11 +48,12 @@ def rotary_table(rot_dims: int, base: float, max_pos: int, device) -> torch.Tens
 class StepBatch:
     """Device-side description of one packed step (see csrc/seqmix.hip)."""
     __slots__ = ("ids", "positions", "slot_mapping", "block_tables", "cu_seqlens", "tok_seq", "state_slots",
-                 "num_tokens", "num_seqs", "tiles", "long_chunks")
+                 "num_tokens", "num_seqs", "tiles", "long_chunks", "pair_tiles")
 
     def __init__(self, ids, positions, slot_mapping, block_tables, cu_seqlens, tok_seq, state_slots, tiles=None,
-                 long_chunks=False):
+                 long_chunks=False, pair_tiles=None):
         self.tiles = tiles                            # 16-row query tiles (ops.query_tiles) or None: one wave per row
+        self.pair_tiles = pair_tiles                  # heads -> tiles of 16 (row, head) pairs (ops.pair_tiles), or None
         self.long_chunks = long_chunks                # some chunk holds several tokens (prompts and portions)
         self.ids, self.positions, self.slot_mapping, self.block_tables = ids, positions, slot_mapping, block_tables
         self.cu_seqlens, self.tok_seq, self.state_slots = cu_seqlens, tok_seq, state_slots
@@ -135,16 +136,25 @@ class LatentAttention:
     def __call__(self, proj: torch.Tensor, b: StepBatch) -> torch.Tensor:
         s, lw, r = self.s, self.lw, self.r
         col = lambda n: proj[:, lw.seg[n][0]: lw.seg[n][0] + lw.seg[n][1]]     # noqa: E731
-        cache, table = r.latent_cache[self.ci], r.rotary(s.rot_dims, s.rot_base)
+        (cache, cache_t), table = r.latent_cache[self.ci], r.rotary(s.rot_dims, s.rot_base)
         if self.writes:
             ops.latent_kv_write(col("dkv"), lw.dkv_norm, table, b.positions, b.slot_mapping, cache, s.kv_rank, s.rot_dim,
-                                r.eps)
+                                r.eps, cache_t=cache_t)
         q = r.linear(ops.rms_norm_rows(col("dq"), lw.dq_norm, r.eps), lw.uq_w)
         T, hw = q.shape[0], s.dim + s.rot_dim
         # the unrotated query part of every head into the latent space: the keys then are the cached latents
         ql = torch.bmm(q.view(T, s.heads, hw)[:, :, : s.dim].transpose(0, 1), lw.uk_w)
-        ol = ops.latent_window_attn(ql, q, hw, s.dim, cache, b.block_tables, b.tok_seq, b.positions, lw.sink, col("g"),
-                                    table, s.window, s.scale)
+        if cache_t is not None and b.pair_tiles is not None:
+            # the matrix cores: tiles of 16 (row, head) pairs; few tiles (decoded tokens, short prompts) spread
+            # their windows' keys over several workgroups
+            tiles = b.pair_tiles(s.heads)
+            n = min(16, max(s.window // 64, 1), max(1024 // max(int(tiles.shape[0]), 1), 1))
+            ol = ops.latent_window_attn_tiles(ops.latent_q_pack(ql, q, hw, s.dim, s.rot_dim, table, b.positions), cache,
+                                              cache_t, b.block_tables, tiles, b.positions, lw.sink, col("g"), s.window,
+                                              s.scale, num_splits=n)
+        else:
+            ol = ops.latent_window_attn(ql, q, hw, s.dim, cache, b.block_tables, b.tok_seq, b.positions, lw.sink, col("g"),
+                                        table, s.window, s.scale)
         o = torch.bmm(ol, lw.uv_t)                      # [heads, tokens, vdim]
         return r.linear(o.transpose(0, 1).reshape(T, s.heads * s.vdim), lw.o_w)
 
@@ -244,8 +254,12 @@ class HybridRunner(ModelRunner):
             else:
                 A = L.lattn
                 if A.kv_from is None:
-                    self.latent_cache.append(torch.zeros(self.num_blocks, BLOCK_SIZE, A.kv_rank + A.rot_dim, dtype=dtype,
-                                                         device=dev))
+                    # the latent pages, token-major with the rotated key part; where the matrix-core attention
+                    # covers the sizes, the latent once more, channel-major
+                    self.latent_cache.append((
+                        torch.zeros(self.num_blocks, BLOCK_SIZE, A.kv_rank + A.rot_dim, dtype=dtype, device=dev),
+                        torch.zeros(self.num_blocks, A.kv_rank, BLOCK_SIZE, dtype=dtype, device=dev)
+                        if ops.latent_tiles_ok(dtype, A.kv_rank, A.rot_dim) else None))
                     latent_of[li] = len(self.latent_cache) - 1
                 self.mixers.append(LatentAttention(A, lw, self, latent_of[li if A.kv_from is None else A.kv_from],
                                                    A.kv_from is None))
@@ -290,6 +304,8 @@ class HybridRunner(ModelRunner):
         widest = max([L.attn.heads * L.attn.vdim for L in spec.layers if L.attn is not None] + [0])
         self._attn_partial = torch.empty(max(self.MAX_KEY_SPLITS * B * widest, 4), dtype=torch.float32, device=dev)
         self.layer_trace = None                       # a list: _forward appends the residual after every layer run
+        self._pair_tiles = {}                         # of the step at hand: heads -> device tiles
+        self._dec_pairs = {}                          # of a decode step of max_num_seqs rows: heads -> device tiles
 
     # ------------------------------------------------------------------ #
     def rotary(self, rot_dims: int, base: float) -> torch.Tensor:
@@ -297,6 +313,19 @@ class HybridRunner(ModelRunner):
         if key not in self._rotary:
             self._rotary[key] = rotary_table(rot_dims, base, self.max_blocks * BLOCK_SIZE, self.device)
         return self._rotary[key]
+
+    def _decode_pair_tiles(self, heads: int) -> torch.Tensor:
+        """Tiles of (row, head) pairs of a decode step: a row's tiles are adjacent, so the first b rows'
+        tiles are a prefix."""
+        if heads not in self._dec_pairs:
+            cu = np.arange(self.max_num_seqs + 1, dtype=np.int64)
+            self._dec_pairs[heads] = torch.from_numpy(ops.pair_tiles(cu, heads)).to(self.device)
+        return self._dec_pairs[heads]
+
+    def _chunk_pair_tiles(self, heads: int) -> torch.Tensor:
+        if heads not in self._pair_tiles:
+            self._pair_tiles[heads] = torch.from_numpy(ops.pair_tiles(self._step_cu, heads)).to(self.device, non_blocking=True)
+        return self._pair_tiles[heads]
 
     MAX_KEY_SPLITS = 16
 
@@ -315,7 +344,8 @@ class HybridRunner(ModelRunner):
         return {"partial": torch.empty(need, dtype=torch.float32, device=self.device), "num_splits": n}
 
     def kv_cache_bytes_per_block(self) -> int:
-        return sum(t[0].numel() * t.element_size() for t in self.k_cache + self.v_cache + self.latent_cache)
+        pages = self.k_cache + self.v_cache + [t for pair in self.latent_cache for t in pair if t is not None]
+        return sum(t[0].numel() * t.element_size() for t in pages)
 
     def state_bytes_per_slot(self) -> int:
         return sum(t[0].numel() * t.element_size() for t in self.conv_state + self.rec_state)
@@ -450,7 +480,8 @@ class HybridRunner(ModelRunner):
     # ------------------------------------------------------------------ #
     def _decode_body(self, b: int) -> None:
         batch = StepBatch(self.ids[:b], self.positions[:b], self.slots[:b], self.block_tables[:b],
-                          self._dec_cu[:b + 1], self._dec_seq[:b], self.row_extra[:b], self._dec_tiles[:b])
+                          self._dec_cu[:b + 1], self._dec_seq[:b], self.row_extra[:b], self._dec_tiles[:b],
+                          pair_tiles=lambda heads: self._decode_pair_tiles(heads)[: b * (-(-heads // 16))])
         resid = self._forward(batch)
         self._logits(resid, out=self.logits_rows[:b])
         self.greedy(self.logits[:b], self.next_ids[:b], ids_out=self.ids[:b])
@@ -466,6 +497,7 @@ class HybridRunner(ModelRunner):
         self._step_state_slots = np.asarray(state_slots, dtype=np.int32)
         # rows go to the matrix cores in tiles of up to 16 rows of one chunk
         self._step_tiles = ops.query_tiles(cu_seqlens)
+        self._step_cu, self._pair_tiles = np.asarray(cu_seqlens, dtype=np.int64), {}
         self._step_long = int(max_q_len) > 1
         if logit_rows is None:
             return super().run_prefill(token_ids, positions, slot_mapping, block_tables, cu_seqlens, context_lens,
@@ -489,7 +521,7 @@ class HybridRunner(ModelRunner):
         slots = torch.from_numpy(self._step_state_slots).to(self.device, non_blocking=True)
         tiles = torch.from_numpy(self._step_tiles).to(self.device, non_blocking=True)
         return self._forward(StepBatch(token_ids, positions, slot_mapping, block_tables.contiguous(), cu_seqlens,
-                                       tok_seq, slots, tiles, self._step_long))
+                                       tok_seq, slots, tiles, self._step_long, pair_tiles=self._chunk_pair_tiles))
 
     def prefill(self, token_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor,
                 block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,

@@ -64,7 +64,9 @@ def plan_num_blocks(args: EngineArgs, cfg: ModelConfig, tp_size: int, num_layers
         runs = [cfg.hybrid.layers[i] for i, _ in cfg.hybrid.runs()]
         per_tok = sum(L.attn.kv_heads * (L.attn.dim + L.attn.vdim) for L in runs if L.attn is not None)
         # a latent attention caches its latent and one rotated key part, unless it reads another layer's
-        per_tok += sum(L.lattn.kv_rank + L.lattn.rot_dim for L in runs if L.lattn is not None and L.lattn.kv_from is None)
+        # (in 16 bits the latent twice: token-major for the scores, channel-major for the weighted sum)
+        per_tok += sum((1 if elem_size == 4 else 2) * L.lattn.kv_rank + L.lattn.rot_dim for L in runs
+                       if L.lattn is not None and L.lattn.kv_from is None)
         per_block = max(per_tok * BLOCK_SIZE * elem_size, 1)
     blocks_per_seq = (max_model_len + BLOCK_SIZE - 1) // BLOCK_SIZE
     want = args.max_num_seqs * blocks_per_seq + 1

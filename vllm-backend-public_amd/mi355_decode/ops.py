@@ -1272,19 +1272,89 @@ def tanh_rows(x: torch.Tensor):
 
 
 def latent_kv_write(x: torch.Tensor, norm_weight: torch.Tensor, cos_sin: torch.Tensor, positions: torch.Tensor,
-                    slot_mapping: torch.Tensor, cache: torch.Tensor, rank: int, rot: int, eps: float):
+                    slot_mapping: torch.Tensor, cache: torch.Tensor, rank: int, rot: int, eps: float,
+                    cache_t: torch.Tensor | None = None):
     """x [tokens, rank + rot] (a column slice is fine): the first rank columns RMS-normed with norm_weight
     (float32), the last rot rotated by the table cos_sin [max_pos, rot_dims], both into the row's slot of
-    cache [blocks, 16, rank + rot]."""
+    cache [blocks, 16, rank + rot]; the latent also into cache_t [blocks, rank, 16] if given."""
     dt = _dt3(x, "x")
     T = x.shape[0]
     if cache.dim() != 3 or tuple(cache.shape[1:]) != (BLOCK_SIZE, rank + rot) or not cache.is_contiguous():
         raise ValueError("latent pages must be contiguous [blocks, 16, rank + rot]")
-    check(lib.mi355_latent_kv_write(_same(cache, x, "cache"), x.data_ptr(), _cols(x, "x", rank + rot),
+    if cache_t is not None and (tuple(cache_t.shape) != (cache.shape[0], rank, BLOCK_SIZE) or not cache_t.is_contiguous()):
+        raise ValueError("the channel-major latent pages must be contiguous [blocks, rank, 16]")
+    check(lib.mi355_latent_kv_write(_same(cache, x, "cache"), None if cache_t is None else _same(cache_t, x, "cache_t"),
+                                    x.data_ptr(), _cols(x, "x", rank + rot),
                                     _f32(norm_weight, "norm_weight", rank), _f32(cos_sin, "cos_sin") or x.data_ptr(),
                                     max(cos_sin.shape[0], 1), _idx(positions, "positions", torch.int64, T),
                                     _idx(slot_mapping, "slot_mapping", torch.int64, T), T, rank, rot, cos_sin.shape[1],
                                     float(eps), dt, _stream()))
+
+
+def pair_tiles(cu_seqlens, num_heads: int) -> "np.ndarray":
+    """(chunk, first pair, pairs <= 16) for every tile of 16 consecutive (packed row, head) pairs of a
+    packed batch, pair number = row * num_heads + head, from the host copy of cu_seqlens: the work
+    list of the matrix-core latent attention."""
+    import numpy as np
+    cu = np.asarray(cu_seqlens, dtype=np.int64) * num_heads
+    out = []
+    for s in range(len(cu) - 1):
+        first = np.arange(cu[s], cu[s + 1], 16, dtype=np.int64)
+        out.append(np.stack([np.full_like(first, s), first, np.minimum(16, cu[s + 1] - first)], axis=1))
+    return (np.concatenate(out) if out else np.zeros((0, 3))).astype(np.int32).reshape(-1, 3)
+
+
+def latent_tiles_ok(dtype: torch.dtype, rank: int, rot: int) -> bool:
+    """Whether the matrix-core latent attention covers these sizes."""
+    return dtype in (torch.bfloat16, torch.float16) and rank % 16 == 0 and (rank + rot) % 8 == 0 and rank <= 512 \
+        and rank + rot <= 640
+
+
+def latent_q_pack(q_latent: torch.Tensor, q: torch.Tensor, q_head_width: int, q_rot_offset: int, rot: int,
+                  cos_sin: torch.Tensor, positions: torch.Tensor):
+    """[tokens, heads, rank + rot] = q_latent [heads, tokens, rank] | the rotated `rot` columns of q at
+    q_rot_offset of every head: the query as latent_window_attn_tiles reads it."""
+    dt = _dt3(q, "q")
+    H, T, rank = q_latent.shape
+    if q_latent.stride(2) != 1 or q.shape[0] != T:
+        raise ValueError("q_latent must be [heads, tokens, rank] with a contiguous last dim")
+    out = torch.empty(T, H, rank + rot, dtype=q.dtype, device=q.device)
+    check(lib.mi355_latent_q_pack(out.data_ptr(), _same(q_latent, q, "q_latent"), max(q_latent.stride(1), rank),
+                                  max(q_latent.stride(0), rank), q.data_ptr(), _cols(q, "q", H * q_head_width), q_head_width,
+                                  q_rot_offset, _f32(cos_sin, "cos_sin") or q.data_ptr(), max(cos_sin.shape[0], 1),
+                                  _idx(positions, "positions", torch.int64, T), T, H, rank, rot, cos_sin.shape[1], dt,
+                                  _stream()))
+    return out
+
+
+def latent_window_attn_tiles(q_packed: torch.Tensor, cache: torch.Tensor, cache_t: torch.Tensor, block_tables: torch.Tensor,
+                             tiles: torch.Tensor, positions: torch.Tensor, sink: torch.Tensor, gate: torch.Tensor | None,
+                             window: int, scale: float, num_splits: int = 1, out: torch.Tensor | None = None):
+    """The matrix-core form of latent_window_attn: q_packed [tokens, heads, rank + rot] (latent_q_pack),
+    both copies of the latent pages, tiles from pair_tiles.  Returns [heads, tokens, rank]."""
+    dt = _dt16(q_packed, "q_packed")
+    T, H, dq = q_packed.shape
+    rank = cache_t.shape[1]
+    if not q_packed.is_contiguous() or tuple(cache.shape[1:]) != (BLOCK_SIZE, dq) or not cache.is_contiguous() \
+            or tuple(cache_t.shape) != (cache.shape[0], rank, BLOCK_SIZE) or not cache_t.is_contiguous():
+        raise ValueError("q_packed [tokens, heads, rank + rot], pages [blocks, 16, rank + rot] and [blocks, rank, 16]")
+    if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 3 or not tiles.is_contiguous() or not tiles.is_cuda:
+        raise ValueError("tiles must be a contiguous int32 [n, 3] tensor on the GPU")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be contiguous int32 [chunks, max_blocks]")
+    if out is None:
+        out = torch.empty(H, T, rank, dtype=q_packed.dtype, device=q_packed.device)
+    partial = None
+    if num_splits > 1:
+        partial = torch.empty(num_splits * T * H * (rank + 2), dtype=torch.float32, device=q_packed.device)
+    check(lib.mi355_latent_window_attn_tiles(
+        out.data_ptr(), max(out.stride(1), rank), max(out.stride(0), rank), q_packed.data_ptr(),
+        _same(cache, q_packed, "cache"), _same(cache_t, q_packed, "cache_t"), block_tables.data_ptr(), block_tables.shape[1],
+        tiles.data_ptr(), tiles.shape[0], _idx(positions, "positions", torch.int64, T), _f32(sink, "sink", H),
+        None if gate is None else _same(gate, q_packed, "gate"), 0 if gate is None else _cols(gate, "gate", H), T, H, rank,
+        dq - rank, int(window), float(scale), None if partial is None else partial.data_ptr(), int(num_splits), dt,
+        _stream()))
+    return out
 
 
 def latent_window_attn(q_latent: torch.Tensor, q: torch.Tensor, q_head_width: int, q_rot_offset: int, cache: torch.Tensor,
