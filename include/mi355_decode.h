@@ -951,19 +951,23 @@ int32_t mi355_latent_window_attn(void* out, int64_t out_stride, int64_t out_head
  *                     experts' scores (no correction, not renormalised)
  *   moe_sort          routed rows by expert: offsets [experts + 1], perm[position] = row,
  *                     inv[row] = position
- *   moe_gather_rows   xs[position] = x[perm[position] / top]
+ *   moe_gather_rows   xs[position] = x[perm[position] / top] for num_rows positions (pad_to 0); with
+ *                     pad_to > 0, num_rows = experts * pad_to and xs[e * pad_to + j] is the j-th row of
+ *                     expert e, zeros past its count (one batched product over all experts then)
  *   moe_gate_up_rows  act[position] = silu(Wg[e] x[t]) * (Wu[e] x[t]); w_gate_up [experts, 2 ff, width]
  *   moe_down_rows     y[position] = Wd[e] act[position]; w_down [experts, width, ff]
  *   moe_silu_and_mul  out = silu(x[:, :ff]) * x[:, ff:]
- *   moe_combine       out[t] = sum_k weights[t, k] * y[inv[t * top + k]]
+ *   moe_combine       out[t] = sum_k weights[t, k] * y[inv[t * top + k]]; with pad_to > 0, y holds every
+ *                     expert's rows padded to pad_to (ids and offsets locate them)
  */
 int32_t mi355_moe_route(int32_t* ids, float* weights, const float* logits, const float* correction,
                         int64_t num_tokens, int32_t experts, int32_t top, int32_t groups, int32_t keep,
                         void* stream);
 int32_t mi355_moe_sort(int32_t* offsets, int32_t* perm, int32_t* inv, const int32_t* ids,
                        int64_t num_rows, int32_t experts, void* stream);
-int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t* perm, int64_t num_rows,
-                              int32_t top, int32_t width, int32_t dtype, void* stream);
+int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t* perm, const int32_t* offsets,
+                              int32_t pad_to, int64_t num_rows, int32_t top, int32_t width,
+                              int32_t dtype, void* stream);
 int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* w_gate_up, const int32_t* offsets,
                                const int32_t* perm, int32_t experts, int32_t top, int32_t width,
                                int32_t ff, int32_t dtype, void* stream);
@@ -972,6 +976,7 @@ int32_t mi355_moe_down_rows(void* y, const void* act, const void* w_down, const 
 int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_rows, int32_t ff, int32_t dtype,
                                void* stream);
 int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights,
+                          const int32_t* ids, const int32_t* offsets, int32_t pad_to,
                           int64_t num_tokens, int32_t top, int32_t width, int32_t dtype, void* stream);
 
 #ifdef __cplusplus

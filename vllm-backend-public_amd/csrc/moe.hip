@@ -5,7 +5,7 @@
 //                       scores the sum of its two best), and weighted by the score without correction
 //   moe_sort            rows (token, choice) ordered by expert: offsets[E + 1], perm[position] = row,
 //                       inv[row] = position
-//   moe_gather_rows     xs[position] = x[perm[position] / top]
+//   moe_gather_rows     xs[position] = x[perm[position] / top]; or every expert's rows padded to a common count
 //   moe_gate_up_rows    a[position] = silu(Wg[e] x) * (Wu[e] x) for every routed row, one wave per
 //                       (expert, hidden unit) walking that expert's rows: an expert's weights leave HBM once
 //   moe_down_rows       y[position] = Wd[e] a[position], the same way
@@ -70,6 +70,82 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int32_t* __restrict__ ids
   }
 }
 
+// (value, index) maximum over the wave, every lane gets it; ties go to the lower index
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(v, off, 64);
+    const int oi = __shfl_xor(i, off, 64);
+    if (ov > v || (ov == v && oi < i)) { v = ov; i = oi; }
+  }
+}
+
+// The same choice, one wave per token: lane j holds experts j, j + 64, ...; groups are scored by the
+// lanes from the choice scores in LDS; every pick is a maximum over the wave.
+template <int EPL>
+__global__ __launch_bounds__(256) void moe_route_wave_kernel(int32_t* __restrict__ ids, float* __restrict__ wts,
+                                                             const float* __restrict__ z, const float* __restrict__ corr,
+                                                             int64_t T, int E, int top, int count, int keep) {
+  __shared__ float ch[4][64 * EPL];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int64_t t = blockIdx.x * 4 + wave;
+  const bool live = t < T;
+  if (!live) t = T - 1;                                 // (every wave reaches the barrier; nothing stored)
+  const float* zr = z + t * E;
+  const float ninf = -__builtin_inff();
+  const int per = E / count;
+  float c[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = lane + 64 * i;
+    c[i] = e < E ? 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + e))) + MI355_LD(float, corr, corr + e) : ninf;
+    ch[wave][e] = c[i];
+  }
+  __syncthreads();
+  if (keep < count) {
+    float gs = ninf;
+    if (lane < count) {
+      float a = ninf, b = ninf;                         // the two largest of the group
+      for (int i = 0; i < per; ++i) {
+        const float v = ch[wave][lane * per + i];
+        if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
+      }
+      gs = per > 1 ? a + b : a;
+    }
+    uint64_t allowed = 0;
+    bool mine = false;                                  // this lane's group has been picked
+    for (int r = 0; r < keep; ++r) {
+      float v = (lane < count && !mine) ? gs : ninf;
+      int g = (lane < count && !mine) ? lane : 0x7FFFFFFF;
+      wave_argmax(v, g);
+      if (lane == g) mine = true;
+      allowed |= 1ull << g;
+    }
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int e = lane + 64 * i;
+      if (e < E && !((allowed >> (e / per)) & 1ull)) c[i] = ninf;
+    }
+  }
+  for (int r = 0; r < top; ++r) {
+    float v = ninf;
+    int e = 0x7FFFFFFF;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) {
+      const int ei = lane + 64 * i;
+      if (ei < E && (c[i] > v || e == 0x7FFFFFFF) && c[i] > ninf) { v = c[i]; e = ei; }
+    }
+    wave_argmax(v, e);
+#pragma unroll
+    for (int i = 0; i < EPL; ++i)
+      if (lane + 64 * i == e) c[i] = ninf;              // taken
+    if (live && lane == 0) {
+      MI355_ST(int32_t, ids, ids + t * top + r, e);
+      MI355_ST(float, wts, wts + t * top + r, 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + e))));
+    }
+  }
+}
+
 // one workgroup: counts, an exclusive prefix, then a position for every row
 __global__ __launch_bounds__(1024) void moe_sort_kernel(int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
                                                         int32_t* __restrict__ inv, const int32_t* __restrict__ ids,
@@ -101,14 +177,25 @@ __global__ __launch_bounds__(1024) void moe_sort_kernel(int32_t* __restrict__ of
   }
 }
 
+// cap 0: xs[position] for every routed row.  cap > 0: every expert's rows padded to cap, xs[e * cap + j]
+// = the j-th row of expert e, zeros past its count (grid: experts * cap rows)
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gather_rows_kernel(typename Elem<T>::S* __restrict__ xs,
                                                               const typename Elem<T>::S* __restrict__ x,
-                                                              const int32_t* __restrict__ perm, int top, int W) {
-  const int64_t p = blockIdx.x;
-  const int64_t t = MI355_LD(int32_t, perm, perm + p) / top;
+                                                              const int32_t* __restrict__ perm,
+                                                              const int32_t* __restrict__ offsets, int cap, int top, int W) {
+  int64_t p = blockIdx.x;
+  bool have = true;
+  if (cap > 0) {
+    const int e = static_cast<int>(p / cap), j = static_cast<int>(p % cap);
+    const int lo = MI355_LD(int32_t, offsets, offsets + e), hi = MI355_LD(int32_t, offsets, offsets + e + 1);
+    have = j < hi - lo;
+    p = lo + j;
+  }
+  const int64_t t = have ? MI355_LD(int32_t, perm, perm + p) / top : 0;
   for (int c = threadIdx.x; c < W; c += blockDim.x)
-    MI355_ST(typename Elem<T>::S, xs, xs + p * W + c, MI355_LD(typename Elem<T>::S, x, x + t * W + c));
+    MI355_ST(typename Elem<T>::S, xs, xs + static_cast<int64_t>(blockIdx.x) * W + c,
+             have ? MI355_LD(typename Elem<T>::S, x, x + t * W + c) : typename Elem<T>::S(0));
 }
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
@@ -236,12 +323,17 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(typename Elem<T>::S* __restrict__ out,
                                                           const typename Elem<T>::S* __restrict__ y,
                                                           const int32_t* __restrict__ inv, const float* __restrict__ wts,
-                                                          int top, int W) {
+                                                          const int32_t* __restrict__ ids,
+                                                          const int32_t* __restrict__ offsets, int cap, int top, int W) {
   const int64_t t = blockIdx.x;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float s = 0.f;
     for (int k = 0; k < top; ++k) {
-      const int64_t p = MI355_LD(int32_t, inv, inv + t * top + k);
+      int64_t p = MI355_LD(int32_t, inv, inv + t * top + k);
+      if (cap > 0) {                                    // y holds every expert's rows padded to cap
+        const int e = MI355_LD(int32_t, ids, ids + t * top + k);
+        p += static_cast<int64_t>(e) * cap - MI355_LD(int32_t, offsets, offsets + e);
+      }
       s += MI355_LD(float, wts, wts + t * top + k) * MI355_LDF(T, y, y + p * W + c);
     }
     MI355_STF(T, out, out + t * W + c, s);
@@ -265,9 +357,19 @@ extern "C" int32_t mi355_moe_route(int32_t* ids, float* weights, const float* lo
                 "moe_route: at most %d chosen experts and %d groups; the kept groups must hold the %d chosen", kMaxTop,
                 kMaxGroups, top);
   if (num_tokens == 0) return MI355_OK;
-  hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((num_tokens + 63) / 64)), dim3(64), 0,
-                     static_cast<hipStream_t>(stream), ids, weights, logits, correction, num_tokens, experts, top, groups,
-                     keep);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 wgrid(static_cast<unsigned>((num_tokens + 3) / 4));
+#define MI355_ROUTE(EPL)                                                                                            \
+  hipLaunchKernelGGL((moe_route_wave_kernel<EPL>), wgrid, dim3(256), 0, s, ids, weights, logits, correction,        \
+                     num_tokens, experts, top, groups, keep)
+  if (experts <= 64) MI355_ROUTE(1);
+  else if (experts <= 128) MI355_ROUTE(2);
+  else if (experts <= 256) MI355_ROUTE(4);
+  else if (experts <= 512) MI355_ROUTE(8);
+  else                                                  // one thread per token
+    hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((num_tokens + 63) / 64)), dim3(64), 0, s, ids, weights,
+                       logits, correction, num_tokens, experts, top, groups, keep);
+#undef MI355_ROUTE
   return check_launch("moe_route");
 }
 
@@ -281,16 +383,18 @@ extern "C" int32_t mi355_moe_sort(int32_t* offsets, int32_t* perm, int32_t* inv,
   return check_launch("moe_sort");
 }
 
-extern "C" int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t* perm, int64_t num_rows, int32_t top,
-                                         int32_t width, int32_t dtype, void* stream) {
+extern "C" int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t* perm, const int32_t* offsets,
+                                         int32_t pad_to, int64_t num_rows, int32_t top, int32_t width, int32_t dtype,
+                                         void* stream) {
   MI355_REQUIRE(xs && x && perm, MI355_ERR_INVALID, "moe_gather_rows: null pointer");
-  MI355_REQUIRE(num_rows >= 0 && top > 0 && width > 0, MI355_ERR_INVALID, "moe_gather_rows: sizes");
+  MI355_REQUIRE(num_rows >= 0 && top > 0 && width > 0 && pad_to >= 0 && (pad_to == 0 || offsets != nullptr), MI355_ERR_INVALID,
+                "moe_gather_rows: sizes");
   REQ_DTYPE(dtype);
   if (num_rows == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_gather_rows_kernel<TT>), dim3(num_rows), dim3(256), 0, s,
                                                   static_cast<Elem<TT>::S*>(xs), static_cast<const Elem<TT>::S*>(x), perm,
-                                                  top, width));
+                                                  offsets, pad_to, top, width));
   return check_launch("moe_gather_rows");
 }
 
@@ -351,15 +455,17 @@ extern "C" int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_
   return check_launch("moe_silu_and_mul");
 }
 
-extern "C" int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights,
-                                     int64_t num_tokens, int32_t top, int32_t width, int32_t dtype, void* stream) {
+extern "C" int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights, const int32_t* ids,
+                                     const int32_t* offsets, int32_t pad_to, int64_t num_tokens, int32_t top, int32_t width,
+                                     int32_t dtype, void* stream) {
   MI355_REQUIRE(out && y && inv && weights, MI355_ERR_INVALID, "moe_combine: null pointer");
-  MI355_REQUIRE(num_tokens >= 0 && top > 0 && width > 0, MI355_ERR_INVALID, "moe_combine: sizes");
+  MI355_REQUIRE(num_tokens >= 0 && top > 0 && width > 0 && pad_to >= 0 && (pad_to == 0 || (ids && offsets)), MI355_ERR_INVALID,
+                "moe_combine: sizes");
   REQ_DTYPE(dtype);
   if (num_tokens == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_combine_kernel<TT>), dim3(num_tokens), dim3(256), 0, s,
                                                   static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(y), inv,
-                                                  weights, top, width));
+                                                  weights, ids, offsets, pad_to, top, width));
   return check_launch("moe_combine");
 }

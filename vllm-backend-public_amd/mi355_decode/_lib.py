@@ -127,11 +127,11 @@ def _load() -> ctypes.CDLL:
                                            I64, I32, I32, I32, I32, I32, F, I32, P]),
         "mi355_moe_route": (I32, [P, P, P, P, I64, I32, I32, I32, I32, P]),
         "mi355_moe_sort": (I32, [P, P, P, P, I64, I32, P]),
-        "mi355_moe_gather_rows": (I32, [P, P, P, I64, I32, I32, I32, P]),
+        "mi355_moe_gather_rows": (I32, [P, P, P, P, I32, I64, I32, I32, I32, P]),
         "mi355_moe_gate_up_rows": (I32, [P, P, P, P, P, I32, I32, I32, I32, I32, P]),
         "mi355_moe_down_rows": (I32, [P, P, P, P, I32, I32, I32, I32, P]),
         "mi355_moe_silu_and_mul": (I32, [P, P, I64, I32, I32, P]),
-        "mi355_moe_combine": (I32, [P, P, P, P, I64, I32, I32, I32, P]),
+        "mi355_moe_combine": (I32, [P, P, P, P, P, P, I32, I64, I32, I32, I32, P]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing

@@ -180,13 +180,11 @@ class MoEFeedForward:
             counts = offsets[1:] - offsets[:-1]
             cap = -(-int(counts.max()) // 16) * 16
             if s.experts * cap <= 2 * rows:
-                at = offsets[:-1].long()[:, None] + torch.arange(cap, device=h.device)[None, :]
-                tok = perm.long()[at.clamp_(max=rows - 1).view(-1)] // s.top      # past an expert's count: some row, unused
-                gu = torch.bmm(h.index_select(0, tok).view(s.experts, cap, -1), lw.gate_up_w.transpose(1, 2))
-                act = ops.moe_silu_and_mul(gu.view(s.experts * cap, 2 * s.ff))
+                xp = ops.moe_gather_rows(h, perm, rows, s.top, offsets=offsets, pad_to=cap)
+                gu = torch.bmm(xp.view(s.experts, cap, -1), lw.gate_up_w.transpose(1, 2)).view(s.experts * cap, 2 * s.ff)
+                act = ops.silu_and_mul(gu) if h.dtype != torch.float32 and s.ff % 8 == 0 else ops.moe_silu_and_mul(gu)
                 y = torch.bmm(act.view(s.experts, cap, s.ff), lw.down_w.transpose(1, 2)).view(s.experts * cap, -1)
-                e = ids.view(-1).long()
-                inv = (inv[:rows].long() + e * cap - offsets.long()[e]).to(torch.int32)
+                return ops.moe_combine(y, inv, wts, T, s.top, ids=ids, offsets=offsets, pad_to=cap)
             else:
                 xs = ops.moe_gather_rows(h, perm, rows, s.top)
                 off = offsets.tolist()

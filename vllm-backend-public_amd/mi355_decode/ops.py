@@ -1413,13 +1413,18 @@ def moe_sort(ids: torch.Tensor, experts: int):
     return offsets, perm, inv
 
 
-def moe_gather_rows(x: torch.Tensor, perm: torch.Tensor, rows: int, top: int):
+def moe_gather_rows(x: torch.Tensor, perm: torch.Tensor, rows: int, top: int, offsets: torch.Tensor | None = None,
+                    pad_to: int = 0):
+    """The routed rows of x in expert order [rows, width]; with pad_to > 0 every expert's rows padded
+    with zero rows to pad_to: [experts * pad_to, width]."""
     dt = _dt3(x, "x")
     if not x.is_contiguous():
         raise ValueError("x must be contiguous")
-    xs = torch.empty(rows, x.shape[1], dtype=x.dtype, device=x.device)
-    check(lib.mi355_moe_gather_rows(xs.data_ptr(), x.data_ptr(), _idx(perm, "perm", torch.int32, rows), rows, int(top),
-                                    x.shape[1], dt, _stream()))
+    n = rows if pad_to <= 0 else (offsets.numel() - 1) * pad_to
+    xs = torch.empty(n, x.shape[1], dtype=x.dtype, device=x.device)
+    check(lib.mi355_moe_gather_rows(xs.data_ptr(), x.data_ptr(), _idx(perm, "perm", torch.int32, rows),
+                                    None if pad_to <= 0 else _idx(offsets, "offsets", torch.int32), max(int(pad_to), 0), n,
+                                    int(top), x.shape[1], dt, _stream()))
     return xs
 
 
@@ -1457,13 +1462,18 @@ def moe_silu_and_mul(x: torch.Tensor):
     return out
 
 
-def moe_combine(y: torch.Tensor, inv: torch.Tensor, weights: torch.Tensor, num_tokens: int, top: int):
-    """out[t] = sum_k weights[t, k] * y[inv[t * top + k]]."""
+def moe_combine(y: torch.Tensor, inv: torch.Tensor, weights: torch.Tensor, num_tokens: int, top: int,
+                ids: torch.Tensor | None = None, offsets: torch.Tensor | None = None, pad_to: int = 0):
+    """out[t] = sum_k weights[t, k] * y[inv[t * top + k]]; with pad_to > 0, y holds every expert's rows
+    padded to pad_to (moe_gather_rows) and ids / offsets locate them."""
     dt = _dt3(y, "y")
     if not y.is_contiguous():
         raise ValueError("y must be contiguous")
     out = torch.empty(num_tokens, y.shape[1], dtype=y.dtype, device=y.device)
+    pad = max(int(pad_to), 0)
     check(lib.mi355_moe_combine(out.data_ptr(), y.data_ptr(), _idx(inv, "inv", torch.int32, num_tokens * top),
-                                _f32(weights, "weights", num_tokens * top), num_tokens, int(top), y.shape[1], dt,
-                                _stream()))
+                                _f32(weights, "weights", num_tokens * top),
+                                None if pad == 0 else _idx(ids, "ids", torch.int32, num_tokens * top),
+                                None if pad == 0 else _idx(offsets, "offsets", torch.int32), pad, num_tokens, int(top),
+                                y.shape[1], dt, _stream()))
     return out
