@@ -845,9 +845,10 @@ int32_t mi355_gated_delta_rule(float* o, const void* qkv, int64_t stride, int32_
  *     u = k / sqrt(sum(k^2) + 1e-6)
  * r / k / v / decay / rate are [tokens, heads * head_dim] activations (column slices are fine), the
  * biases fp32 [heads * head_dim]; everything past the projections is fp32.  o is fp32
- * [tokens, heads, head_dim].  workspace: mi355_general_delta_rule_workspace(...) floats.
- * long_chunks 1: state rows split over adjacent lanes (chunks of many tokens); 0: one state column
- * per lane (chunks of a token or two: decode).  Both give the same numbers for any chunk.
+ * [tokens, heads, head_dim].  long_chunks 1: state rows split over adjacent lanes, per-token vectors
+ * prepared for all tokens first into workspace (mi355_general_delta_rule_workspace(...) floats): chunks
+ * of many tokens.  long_chunks 0: one state column per lane, no workspace (may be null): chunks of a
+ * token or two (decode).  Both give the same numbers for any chunk.
  */
 int64_t mi355_general_delta_rule_workspace(int64_t num_tokens, int32_t num_heads, int32_t head_dim);
 int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_stride, const void* k,

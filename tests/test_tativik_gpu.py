@@ -174,10 +174,14 @@ def test_general_delta_rule_whole_portions_and_single_tokens(H, d):
     x = torch.randn(T, 5, H * d, generator=g)
     w0, ab = torch.randn(H * d, generator=g), torch.randn(H * d, generator=g) * 0.5
     ref = _gdelta_ref(x, w0, ab, H, d)
+    x16 = x.to(torch.bfloat16)
+    ref16 = _gdelta_ref(x16.float(), w0, ab, H, d)
     for cuts in ([T], [1] * T, [2, 3, 1, 17, 2, 16]):
         for long_chunks in (True, False):                   # state rows split over lanes; one state column per lane
             got, _ = _gdelta_in_cuts(x, w0, ab, cuts, H, d, long_chunks=long_chunks)
             assert (got - ref).abs().max() <= 3e-5 * ref.abs().max(), (cuts, long_chunks)
+            got, _ = _gdelta_in_cuts(x16, w0, ab, cuts, H, d, long_chunks=long_chunks)     # 16-bit inputs, fp32 inside
+            assert (got - ref16).abs().max() <= 3e-5 * ref16.abs().max(), (cuts, long_chunks, "bfloat16")
 
 
 def test_general_delta_rule_keeps_a_far_write_removes_it_along_its_key_and_forgets_it_with_decay():
@@ -391,14 +395,15 @@ def test_routing_groups_corrections_and_negative_choice_scores():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("T", [1, 5, 300])
-def test_expert_products_by_rows_and_by_expert_matrices(dtype, T):
+@pytest.mark.parametrize("W,F", [(72, 40), (96, 64)])           # the second: sizes that the matrix-core row kernels cover in 16 bits
+def test_expert_products_by_rows_and_by_expert_matrices(dtype, T, W, F):
     """The mixture through the runner's feed-forward object: few rows take the per-row kernels, many
     rows one library product per expert; both against the restatement."""
     from types import SimpleNamespace
     from mi355_decode.config import MoESpec
     from mi355_decode.hybrid_runner import MoEFeedForward
     g = torch.Generator().manual_seed(T)
-    W, E, F, top = 72, 6, 40, 3
+    E, top = 6, 3
     wt = {"router": torch.randn(E, W, generator=g) * W ** -0.5, "correction": torch.randn(E, generator=g) * 0.3}
     for e in range(E):
         wt[f"e{e}.gate"], wt[f"e{e}.up"] = torch.randn(F, W, generator=g) * W ** -0.5, torch.randn(F, W, generator=g) * W ** -0.5

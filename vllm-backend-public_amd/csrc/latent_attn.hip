@@ -509,7 +509,8 @@ extern "C" int32_t mi355_latent_window_attn_tiles(void* out, int64_t out_stride,
   const int64_t pairs = num_tokens * num_heads;
   float* part_acc = split ? partial : nullptr;
   float* part_ml = split ? partial + static_cast<int64_t>(num_splits) * pairs * rank : nullptr;
-  const int waves = num_tiles < 4 ? num_tiles : 4;
+  // few tiles (decoded tokens): one wave per workgroup, so that they spread over the compute units
+  const int waves = static_cast<int64_t>(num_tiles) * num_splits <= 2048 ? 1 : 4;
   const dim3 grid(static_cast<unsigned>((num_tiles + waves - 1) / waves), 1u, static_cast<unsigned>(num_splits));
   const dim3 block(64u * static_cast<unsigned>(waves));
   const float scale2 = scale * kLog2e;

@@ -8,7 +8,8 @@
 //   moe_gather_rows     xs[position] = x[perm[position] / top]; or every expert's rows padded to a common count
 //   moe_gate_up_rows    a[position] = silu(Wg[e] x) * (Wu[e] x) for every routed row, one wave per
 //                       (expert, hidden unit) walking that expert's rows: an expert's weights leave HBM once
-//   moe_down_rows       y[position] = Wd[e] a[position], the same way
+//   moe_down_rows       y[position] = Wd[e] a[position], the same way; both on the matrix cores where the
+//                       sizes allow (16-bit storage, widths multiples of 32 / 16)
 //   moe_silu_and_mul    a = silu(gu[:, :F]) * gu[:, F:] (any storage type)
 //   moe_combine         out[t] = sum_k weight[t, k] * y[inv[t * top + k]]
 // Routing, scores and the weighted sum are fp32; activations and expert weights are stored in the
@@ -306,6 +307,64 @@ __global__ __launch_bounds__(256) void moe_down_rows_kernel(typename Elem<T>::S*
   }
 }
 
+// The same two products on the matrix cores (16-bit storage): a wave streams 16 weight rows of one
+// expert once and multiplies them into that expert's routed rows, 16 at a time -- the rows are the
+// columns of a 16 x 16 x 32 product, so a decode step's handful of rows per expert costs one pass
+// over the expert's weights and one matrix instruction per 32 weights of a row.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(uint16_t* __restrict__ a, const uint16_t* __restrict__ x,
+                                                               const uint16_t* __restrict__ w_gate_up,
+                                                               const int32_t* __restrict__ offsets,
+                                                               const int32_t* __restrict__ perm, int top, int W, int F) {
+  const int e = blockIdx.y, lane = threadIdx.x & 63, li = lane & 15, kk = lane >> 4;
+  const int f0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16;
+  if (f0 >= F) return;
+  const int lo = MI355_LD(int32_t, offsets, offsets + e), hi = MI355_LD(int32_t, offsets, offsets + e + 1);
+  const uint16_t* wg = w_gate_up + (static_cast<int64_t>(e) * 2 * F + f0 + li) * W + 8 * kk;
+  const uint16_t* wu = wg + static_cast<int64_t>(F) * W;
+  for (int p0 = lo; p0 < hi; p0 += 16) {
+    const int p = p0 + li < hi ? p0 + li : p0;          // columns past the expert's last row: its first row again, not stored
+    const uint16_t* xr = x + static_cast<int64_t>(MI355_LD(int32_t, perm, perm + p) / top) * W + 8 * kk;
+    f32x4 g = f32x4{0.f, 0.f, 0.f, 0.f}, u = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < W; s += 32) {                   // (two chains of products in turn: gate, up)
+      const uint4 b = MI355_LD(uint4, x, xr + s);
+      g = T::mfma(MI355_LD(uint4, w_gate_up, wg + s), b, g);
+      u = T::mfma(MI355_LD(uint4, w_gate_up, wu + s), b, u);
+    }
+    if (p0 + li < hi) {
+      float out[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) out[r] = silu_f(round_f<T>(g[r])) * round_f<T>(u[r]);      // as stored by a product
+      MI355_ST(uint2, a, a + static_cast<int64_t>(p0 + li) * F + f0 + 4 * kk,
+               make_uint2(T::pack2(out[0], out[1]), T::pack2(out[2], out[3])));
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_mfma_kernel(uint16_t* __restrict__ y, const uint16_t* __restrict__ a,
+                                                            const uint16_t* __restrict__ w_down,
+                                                            const int32_t* __restrict__ offsets, int W, int F) {
+  const int e = blockIdx.y, lane = threadIdx.x & 63, li = lane & 15, kk = lane >> 4;
+  const int c0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16;
+  if (c0 >= W) return;
+  const int lo = MI355_LD(int32_t, offsets, offsets + e), hi = MI355_LD(int32_t, offsets, offsets + e + 1);
+  const uint16_t* wd = w_down + (static_cast<int64_t>(e) * W + c0 + li) * F + 8 * kk;
+  for (int p0 = lo; p0 < hi; p0 += 16) {
+    const uint16_t* ar = a + static_cast<int64_t>(p0 + li < hi ? p0 + li : p0) * F + 8 * kk;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f}, acc2 = f32x4{0.f, 0.f, 0.f, 0.f};     // two chains of products in turn
+    for (int s = 0; s < F; s += 64) {
+      acc = T::mfma(MI355_LD(uint4, w_down, wd + s), MI355_LD(uint4, a, ar + s), acc);
+      if (s + 32 < F) acc2 = T::mfma(MI355_LD(uint4, w_down, wd + s + 32), MI355_LD(uint4, a, ar + s + 32), acc2);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc[r] += acc2[r];
+    if (p0 + li < hi)
+      MI355_ST(uint2, y, y + static_cast<int64_t>(p0 + li) * W + c0 + 4 * kk,
+               make_uint2(T::pack2(acc[0], acc[1]), T::pack2(acc[2], acc[3])));
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_silu_and_mul_kernel(typename Elem<T>::S* __restrict__ out,
                                                                const typename Elem<T>::S* __restrict__ x, int64_t rows,
@@ -407,6 +466,16 @@ extern "C" int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* 
   REQ_DTYPE(dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>((ff + 3) / 4), static_cast<unsigned>(experts));
+  if (dtype != MI355_F32 && width % 32 == 0 && ff % 16 == 0 && aligned16(x) && aligned16(w_gate_up) && aligned16(act)) {
+    const dim3 mgrid(static_cast<unsigned>((ff / 16 + 3) / 4), static_cast<unsigned>(experts));
+    if (dtype == MI355_BF16)
+      hipLaunchKernelGGL((moe_gate_up_mfma_kernel<BF16>), mgrid, dim3(256), 0, s, static_cast<uint16_t*>(act),
+                         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w_gate_up), offsets, perm, top, width, ff);
+    else
+      hipLaunchKernelGGL((moe_gate_up_mfma_kernel<F16>), mgrid, dim3(256), 0, s, static_cast<uint16_t*>(act),
+                         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w_gate_up), offsets, perm, top, width, ff);
+    return check_launch("moe_gate_up_rows (matrix cores)");
+  }
   const bool vec = dtype != MI355_F32 && width % 8 == 0 && aligned16(x) && aligned16(w_gate_up);
   MI355_DISPATCH_DTYPE3(dtype, {
     if (vec)
@@ -428,6 +497,16 @@ extern "C" int32_t mi355_moe_down_rows(void* y, const void* act, const void* w_d
   REQ_DTYPE(dtype);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>((width + 3) / 4), static_cast<unsigned>(experts));
+  if (dtype != MI355_F32 && ff % 32 == 0 && width % 16 == 0 && aligned16(act) && aligned16(w_down) && aligned16(y)) {
+    const dim3 mgrid(static_cast<unsigned>((width / 16 + 3) / 4), static_cast<unsigned>(experts));
+    if (dtype == MI355_BF16)
+      hipLaunchKernelGGL((moe_down_mfma_kernel<BF16>), mgrid, dim3(256), 0, s, static_cast<uint16_t*>(y),
+                         static_cast<const uint16_t*>(act), static_cast<const uint16_t*>(w_down), offsets, width, ff);
+    else
+      hipLaunchKernelGGL((moe_down_mfma_kernel<F16>), mgrid, dim3(256), 0, s, static_cast<uint16_t*>(y),
+                         static_cast<const uint16_t*>(act), static_cast<const uint16_t*>(w_down), offsets, width, ff);
+    return check_launch("moe_down_rows (matrix cores)");
+  }
   const bool vec = dtype != MI355_F32 && ff % 8 == 0 && aligned16(act) && aligned16(w_down);
   MI355_DISPATCH_DTYPE3(dtype, {
     if (vec)

@@ -745,14 +745,19 @@ __global__ __launch_bounds__(64) void general_delta_rule_kernel(
 }
 
 // The same recurrence for chunks of one or two tokens (decode): one wave per (chunk, head, 64 value
-// channels), lane j owns column j of S in registers, so a state row is one coalesced load; the
-// per-token vectors come from the prepared rows (every lane reads the same address).
+// channels), lane j owns column j of S in registers, so a state row is one coalesced load.  The wave
+// prepares the token's vectors itself, in LDS (no workspace, one launch); with heads wider than 64
+// the waves of a head each do so.
 template <typename T, int D>
 __global__ __launch_bounds__(64) void general_delta_rule_cols_kernel(
-    float* __restrict__ o, const typename Elem<T>::S* __restrict__ v, int64_t v_stride, const float* __restrict__ ws,
-    int dp, float* __restrict__ state, const int32_t* __restrict__ cu_seqlens, const int64_t* __restrict__ positions,
-    const int32_t* __restrict__ state_slots, int H, int d) {
-  const int s = blockIdx.x, h = blockIdx.y, col = blockIdx.z * 64 + threadIdx.x;
+    float* __restrict__ o, const typename Elem<T>::S* __restrict__ r, int64_t r_stride,
+    const typename Elem<T>::S* __restrict__ k, int64_t k_stride, const typename Elem<T>::S* __restrict__ v, int64_t v_stride,
+    const typename Elem<T>::S* __restrict__ wl, int64_t wl_stride, const float* __restrict__ w0,
+    const typename Elem<T>::S* __restrict__ al, int64_t al_stride, const float* __restrict__ ab, float* __restrict__ state,
+    const int32_t* __restrict__ cu_seqlens, const int64_t* __restrict__ positions, const int32_t* __restrict__ state_slots,
+    int H, int d) {
+  __shared__ float ws[D], us[D], aus[D], ks[D], rs[D];
+  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, col = blockIdx.z * 64 + lane;
   const int64_t cs = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s);
   const int64_t n = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1) - cs;
   if (n <= 0) return;
@@ -764,23 +769,48 @@ __global__ __launch_bounds__(64) void general_delta_rule_cols_kernel(
 #pragma unroll
   for (int i = 0; i < D; ++i) S[i] = (live && !fresh && i < d) ? MI355_LD(float, state, sp + static_cast<int64_t>(i) * d + col) : 0.f;
   for (int64_t t = cs; t < cs + n; ++t) {
-    const float* p = ws + (t * H + h) * 5 * dp;
-    const float vj = live ? MI355_LDF(T, v, v + t * v_stride + static_cast<int64_t>(h) * d + col) : 0.f;
+    const int64_t hd = static_cast<int64_t>(h) * d;
+    float kv[(D + 63) / 64], kk = 0.f;
+#pragma unroll
+    for (int i = 0; i < (D + 63) / 64; ++i) {
+      const int c = lane + 64 * i;
+      kv[i] = c < d ? MI355_LDF(T, k, k + t * k_stride + hd + c) : 0.f;
+      kk += kv[i] * kv[i];
+    }
+    kk = 1.0f / sqrtf(wave_sum(kk) + 1e-6f);
+    __syncthreads();                                    // the previous token's reads of the vectors are done
+#pragma unroll
+    for (int i = 0; i < (D + 63) / 64; ++i) {
+      const int c = lane + 64 * i;
+      if (c < D) {
+        float w = 1.f, u = 0.f, au = 0.f, rv = 0.f;
+        if (c < d) {
+          u = kv[i] * kk;
+          rv = MI355_LDF(T, r, r + t * r_stride + hd + c);
+          const float zw = MI355_LDF(T, wl, wl + t * wl_stride + hd + c) + MI355_LD(float, w0, w0 + hd + c);
+          w = expf(-0.6065306597126334f / (1.0f + expf(-zw)));
+          const float za = MI355_LDF(T, al, al + t * al_stride + hd + c) + MI355_LD(float, ab, ab + hd + c);
+          au = u / (1.0f + expf(-za));
+        }
+        ws[c] = w, us[c] = u, aus[c] = au, ks[c] = kv[i], rs[c] = rv;
+      }
+    }
+    const float vj = live ? MI355_LDF(T, v, v + t * v_stride + hd + col) : 0.f;
+    __syncthreads();
     float d0 = 0.f, d1 = 0.f;
 #pragma unroll
     for (int i = 0; i < D; i += 2) {
-      d0 += S[i] * MI355_LD(float, ws, p + dp + i);
-      d1 += S[i + 1] * MI355_LD(float, ws, p + dp + i + 1);
+      d0 += S[i] * us[i];
+      d1 += S[i + 1] * us[i + 1];
     }
     const float dot = d0 + d1;
     float o0 = 0.f, o1 = 0.f;
 #pragma unroll
     for (int i = 0; i < D; i += 2) {
-      S[i] = MI355_LD(float, ws, p + i) * S[i] - MI355_LD(float, ws, p + 2 * dp + i) * dot + MI355_LD(float, ws, p + 3 * dp + i) * vj;
-      S[i + 1] = MI355_LD(float, ws, p + i + 1) * S[i + 1] - MI355_LD(float, ws, p + 2 * dp + i + 1) * dot +
-                 MI355_LD(float, ws, p + 3 * dp + i + 1) * vj;
-      o0 += S[i] * MI355_LD(float, ws, p + 4 * dp + i);
-      o1 += S[i + 1] * MI355_LD(float, ws, p + 4 * dp + i + 1);
+      S[i] = ws[i] * S[i] - aus[i] * dot + ks[i] * vj;
+      S[i + 1] = ws[i + 1] * S[i + 1] - aus[i + 1] * dot + ks[i + 1] * vj;
+      o0 += S[i] * rs[i];
+      o1 += S[i + 1] * rs[i + 1];
     }
     if (live) MI355_ST(float, o, o + (t * H + h) * d + col, o0 + o1);
   }
@@ -1073,7 +1103,7 @@ extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_s
                                             int32_t num_heads, int32_t head_dim, int64_t num_tokens, int32_t long_chunks,
                                             float* workspace, int64_t workspace_floats, int32_t dtype, void* stream) {
   MI355_REQUIRE(o && r && k && v && decay && decay_bias && rate && rate_bias && state && cu_seqlens && positions &&
-                    state_slots && workspace,
+                    state_slots && (workspace || !long_chunks),
                 MI355_ERR_INVALID, "general_delta_rule: null pointer");
   MI355_REQUIRE(num_seqs >= 0 && num_tokens >= 0 && num_heads > 0 && head_dim > 0, MI355_ERR_INVALID,
                 "general_delta_rule: sizes");
@@ -1085,22 +1115,34 @@ extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_s
   REQ_DTYPE(dtype);
   if (num_seqs == 0 || num_tokens == 0) return MI355_OK;
   const int64_t dp = general_delta_dp(head_dim);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (!long_chunks) {
+    // the form for chunks of a token or two: one state column per lane, no workspace
+    const dim3 cgrid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>((head_dim + 63) / 64));
+#define MI355_GCOLS(D)                                                                                                 \
+  hipLaunchKernelGGL((general_delta_rule_cols_kernel<TT, D>), cgrid, dim3(64), 0, s, o, static_cast<const E*>(r),     \
+                     r_stride, static_cast<const E*>(k), k_stride, static_cast<const E*>(v), v_stride,                 \
+                     static_cast<const E*>(decay), decay_stride, decay_bias, static_cast<const E*>(rate), rate_stride, \
+                     rate_bias, state, cu_seqlens, positions, state_slots, num_heads, head_dim)
+    MI355_DISPATCH_DTYPE3(dtype, {
+      typedef Elem<TT>::S E;
+      if (dp == 32) MI355_GCOLS(32);
+      else if (dp == 64) MI355_GCOLS(64);
+      else if (dp == 128) MI355_GCOLS(128);
+      else MI355_GCOLS(256);
+    });
+#undef MI355_GCOLS
+    return check_launch("general_delta_rule (one column per lane)");
+  }
   const int64_t need = mi355_general_delta_rule_workspace(num_tokens, num_heads, head_dim);
   MI355_REQUIRE(workspace_floats >= need && aligned16(workspace), MI355_ERR_INVALID,
                 "general_delta_rule: workspace of %lld floats, %lld needed, 16-byte aligned",
                 static_cast<long long>(workspace_floats), static_cast<long long>(need));
-  hipStream_t s = static_cast<hipStream_t>(stream);
   const int lanes = head_dim <= 32 ? 8 : 16;
   const int cols = 64 / lanes;
   const dim3 pgrid(static_cast<unsigned>(num_tokens), static_cast<unsigned>(num_heads));
   const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads),
                   static_cast<unsigned>((head_dim + cols - 1) / cols));
-  // the form for chunks of a token or two: one state column per lane
-  const dim3 cgrid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), static_cast<unsigned>((head_dim + 63) / 64));
-#define MI355_GCOLS(D)                                                                                                 \
-  hipLaunchKernelGGL((general_delta_rule_cols_kernel<TT, D>), cgrid, dim3(64), 0, s, o, static_cast<const E*>(v),     \
-                     v_stride, workspace, static_cast<int>(dp), state, cu_seqlens, positions, state_slots, num_heads, \
-                     head_dim)
 #define MI355_GDELTA(TT, R, DR, PF)                                                                                  \
   hipLaunchKernelGGL((general_delta_rule_kernel<TT, R, DR, PF>), grid, dim3(64), 0, s, o,                            \
                      static_cast<const Elem<TT>::S*>(v), v_stride, workspace, state, cu_seqlens, positions,          \
@@ -1111,17 +1153,11 @@ extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_s
                        r_stride, static_cast<const E*>(k), k_stride, static_cast<const E*>(decay), decay_stride,
                        decay_bias, static_cast<const E*>(rate), rate_stride, rate_bias, num_heads, head_dim,
                        static_cast<int>(dp));
-    if (!long_chunks) {
-      if (dp == 32) MI355_GCOLS(32);
-      else if (dp == 64) MI355_GCOLS(64);
-      else if (dp == 128) MI355_GCOLS(128);
-      else MI355_GCOLS(256);
-    } else if (dp == 32) MI355_GDELTA(TT, 8, 4, 4);
+    if (dp == 32) MI355_GDELTA(TT, 8, 4, 4);
     else if (dp == 64) MI355_GDELTA(TT, 16, 4, 4);
     else if (dp == 128) MI355_GDELTA(TT, 16, 8, 2);
     else MI355_GDELTA(TT, 16, 16, 1);
   });
 #undef MI355_GDELTA
-#undef MI355_GCOLS
   return check_launch("general_delta_rule");
 }

@@ -1211,14 +1211,16 @@ def general_delta_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay:
         out = torch.empty(T, num_heads, head_dim, dtype=torch.float32, device=r.device)
     if T == 0:
         return out
-    ws = torch.empty(lib.mi355_general_delta_rule_workspace(T, num_heads, head_dim), dtype=torch.float32, device=r.device)
+    ws = None
+    if long_chunks:
+        ws = torch.empty(lib.mi355_general_delta_rule_workspace(T, num_heads, head_dim), dtype=torch.float32, device=r.device)
     check(lib.mi355_general_delta_rule(
         _f32(out, "out", T * C), r.data_ptr(), _cols(r, "r", C), _same(k, r, "k"), _cols(k, "k", C), _same(v, r, "v"),
         _cols(v, "v", C), _same(decay, r, "decay"), _cols(decay, "decay", C), _f32(decay_bias, "decay_bias", C),
         _same(rate, r, "rate"), _cols(rate, "rate", C), _f32(rate_bias, "rate_bias", C), _f32(state, "state"),
         _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(positions, "positions", torch.int64, T),
-        _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, head_dim, T, int(bool(long_chunks)), ws.data_ptr(),
-        ws.numel(), dt, _stream()))
+        _idx(state_slots, "state_slots", torch.int32, S), S, num_heads, head_dim, T, int(bool(long_chunks)),
+        None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), dt, _stream()))
     return out
 
 
