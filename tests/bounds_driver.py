@@ -129,6 +129,60 @@ def engine_generation():
     return out
 
 
+def sandwich_generation():
+    """A hybrid decoder of the sandwich arrangement (general delta rule, latent attention with shared
+    pages, mixture of experts): prompts in portions, single tokens, a mixed batch, then generation --
+    in bfloat16 (the matrix-core attention and expert kernels) and in float32 (their plain forms)."""
+    from mi355_decode import weights as W
+    from mi355_decode.config import EngineArgs, ModelConfig
+    from mi355_decode.llm import build_engine
+    from mi355_decode.sampling_params import SamplingParams
+    lat = {"heads": 6, "dim": 32, "rot_dim": 16, "vdim": 32, "kv_rank": 64, "q_rank": 48, "mask": {"size": 40},
+           "rot": {"dims": 16, "base": 10000.0}, "scale": 0.15}
+    moe = {"kind": "moe", "expert": {"ff": 64}, "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    cfg = ModelConfig.from_dict({
+        "architecture": "Tativik", "width": 128, "vocab": 300, "norm": {"eps": 1e-6, "groups": 2}, "residual_mult": 0.7,
+        "layers": [{"type": "general_delta", "mixer": {"heads": 2, "dim": 64}, "mlp": moe},
+                   {"type": "latent_attention", "mixer": lat, "mlp": moe},
+                   {"type": "latent_attention", "mixer": dict(lat, heads=3, kv_from=1), "mlp": None},
+                   {"type": "general_delta", "mixer": {"heads": 1, "dim": 40}, "mlp": moe}]})
+    state = W.hybrid_synthetic_state(cfg, seed=3)
+    rng = np.random.default_rng(1)
+    out = []
+    for dtype in ("bfloat16", "float32"):
+        bounds.clear()
+        eng = build_engine(EngineArgs(model="sandwich", dtype=dtype, max_num_seqs=4, max_model_len=256,
+                                      num_gpu_blocks_override=48, gpu_memory_utilization=0.0, max_num_batched_tokens=1 << 20),
+                           state_dict=state, model_config=cfg)
+
+        def run(tag):
+            toks = {r: rng.integers(0, 300, n).tolist() for r, n in (("a", 150), ("b", 37), ("c", 2))}
+            eng.forced_step([(tag + "a", toks["a"][:100], [99]), (tag + "c", toks["c"][:1], [0])])
+            eng.forced_step([(tag + "a", toks["a"][100:102], [1]), (tag + "b", toks["b"][:33], []), (tag + "c", toks["c"][1:], [0])],
+                            [tag + "c"])
+            for i in range(4):
+                eng.forced_step([(tag + "a", toks["a"][102 + i:103 + i], [0]), (tag + "b", toks["b"][33 + i:34 + i], [0])])
+            eng.forced_step([(tag + "a", toks["a"][106:], [])], [tag + "a", tag + "b"])
+            for i, n in enumerate((5, 70, 17)):
+                eng.add_request(f"{tag}g{i}", rng.integers(0, 300, n).tolist(),
+                                SamplingParams(max_tokens=10, temperature=0.0 if i else 0.8, seed=i, ignore_eos=True))
+            n = 0
+            while eng.has_unfinished():
+                n += sum(len(o.new_token_ids) for o in eng.step())
+            return n
+
+        run("warm")
+        n = bounds.sync_allocations(granularity="segment")
+        toks = run("checked")
+        rep = bounds.report()
+        assert rep is None or rep["refused"] == 0, (dtype, rep)
+        out.append(f"{dtype}:{toks} tokens:{n} segments:{rep['unknown_base'] if rep else 0} accesses with an unlisted base")
+        del eng
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
 def sampler_rows():
     """The sampling launch on exactly sized logits (no slack behind the last row), every kind of
     row in one call: greedy, whole-vocabulary draw, top-k / top-p cuts, an all-tied row (the list
@@ -166,4 +220,5 @@ if __name__ == "__main__":
     res["sampler"] = sampler_rows()
     res["rank_steps"] = rank_steps()
     res["engine"] = engine_generation()
+    res["sandwich"] = sandwich_generation()
     print(json.dumps(res))
