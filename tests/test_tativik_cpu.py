@@ -65,6 +65,14 @@ def test_weight_layout_and_page_accounting():
     assert l0.router_w.dtype == torch.float32 and l1.gate_up_w is None and w.embed_norm.shape == (96,)
     # synthetic weights come under the same names
     assert set(W.hybrid_synthetic_state(cfg, seed=0)) == set(st)
+    # a configuration that names neither the query latent's size nor a window: the tensor's shape, no window
+    for L in d["layers"]:
+        L["mixer"].pop("q_rank", None)
+        L["mixer"].pop("mask", None)
+    cfg2 = ModelConfig.from_dict(d)
+    assert cfg2.hybrid.layers[0].lattn.q_rank == 0 and cfg2.hybrid.layers[0].lattn.window >= 1 << 30
+    w2 = W.from_state_dict(cfg2, st, torch.float32, "cpu")
+    assert cfg2.hybrid.layers[0].lattn.q_rank == 24 and torch.equal(w2.layers[0].uq_w, l0.uq_w)
 
 
 def test_restatement_edges_and_cut_invariance():

@@ -550,3 +550,68 @@ def test_greedy_generation_through_the_engine(name, dtype):
         for t in range(steps):
             best = int(torch.argmax(z[t]))
             assert o[t] == best or float(z[t, best] - z[t, o[t]]) <= tol, f"token {t}: {o[t]} vs {best}"
+
+
+def test_served_from_a_model_directory(tmp_path):
+    """The OpenAI server started on a directory with config.json + model.safetensors of this design: the
+    model class chosen by config.json, weights from the checkpoint names, greedy completions by token
+    id against the restatement (margin rule), and a seeded sampled completion through the sampler."""
+    import json
+    import os
+    import signal
+    import socket
+    import subprocess
+    import sys
+    import time
+    from safetensors.torch import save_file
+    from conftest import PKG, ROOT
+    from mi355_decode.harness import BenchClient
+    name = "mix"
+    cfg, w = CONFIGS[name], _weights(name)
+    model_dir = tmp_path / "model"
+    model_dir.mkdir()
+    json.dump(cfg, open(model_dir / "config.json", "w"))
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in w.items()}, str(model_dir / "model.safetensors"))
+    with socket.socket() as s:
+        s.bind(("127.0.0.1", 0))
+        port = s.getsockname()[1]
+    args = ["--model", str(model_dir), "--served-model-name", "sandwich", "--host", "127.0.0.1", "--port", str(port),
+            "--dtype", "float32", "--max-num-seqs", "4", "--max-model-len", "128"]
+    env = dict(os.environ, PYTHONPATH=PKG + os.pathsep + ROOT)
+    log = open(tmp_path / "server.log", "w")
+    proc = subprocess.Popen([sys.executable, "-m", "mi355_decode.entrypoints.openai.api_server"] + args, env=env, stdout=log,
+                            stderr=subprocess.STDOUT, start_new_session=True)
+    url = f"http://127.0.0.1:{port}"
+    try:
+        client = BenchClient(url)
+        t0 = time.time()
+        while True:
+            assert proc.poll() is None, open(tmp_path / "server.log").read()[-3000:]
+            try:
+                if client.health() == 200:
+                    break
+            except Exception:
+                pass
+            assert time.time() - t0 < 240, "server did not become healthy"
+            time.sleep(0.2)
+        post = lambda **body: client.http.post(f"{url}/v1/completions", json={"model": "sandwich", **body})   # noqa: E731
+        prompt, steps = _tokens(name, 21, 5), 12
+        r = post(prompt=prompt, max_tokens=steps, temperature=0, ignore_eos=True, logprobs=0, return_tokens_as_token_ids=True)
+        assert r.status_code == 200, r.text
+        got = [int(t.split(":")[1]) for t in r.json()["choices"][0]["logprobs"]["tokens"]]
+        assert len(got) == steps
+        with torch.no_grad():
+            z = R.forward(w, cfg, prompt + got)[len(prompt) - 1: -1]
+        for t in range(steps):
+            best = int(torch.argmax(z[t]))
+            assert got[t] == best or float(z[t, best] - z[t, got[t]]) <= 2e-3, f"token {t}"
+        draws = [post(prompt=prompt, max_tokens=8, temperature=0.9, top_k=20, seed=7, ignore_eos=True, logprobs=0,
+                      return_tokens_as_token_ids=True).json()["choices"][0]["logprobs"]["tokens"] for _ in range(2)]
+        assert draws[0] == draws[1] and len(draws[0]) == 8
+        assert "synthetic" not in open(tmp_path / "server.log").read()
+    finally:
+        os.killpg(proc.pid, signal.SIGTERM)
+        try:
+            proc.wait(timeout=20)
+        except subprocess.TimeoutExpired:
+            os.killpg(proc.pid, signal.SIGKILL)

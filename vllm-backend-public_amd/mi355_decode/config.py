@@ -92,7 +92,8 @@ class LatentAttnSpec:
     part is one vector shared by all heads, rotation on its first rot_dims coordinates), values of
     vdim; sliding window; a learned sink per head in the softmax denominator; one output gate per
     head.  kv_from: the layer whose cached latent and rotated key this layer reads instead of making
-    its own (None: its own)."""
+    its own (None: its own).  q_rank 0: not in the configuration, the weights' shape gives it; a
+    configuration without a window gets one longer than any sequence."""
     heads: int
     dim: int
     rot_dim: int
@@ -183,7 +184,8 @@ class HybridSpec:
             elif spec["type"] == "latent_attention":
                 rot = m.get("rot") or {}
                 a = LatentAttnSpec(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=int(m["rot_dim"]), vdim=int(m["vdim"]),
-                                   kv_rank=int(m["kv_rank"]), q_rank=int(m["q_rank"]), window=int(m["mask"]["size"]),
+                                   kv_rank=int(m["kv_rank"]), q_rank=int(m.get("q_rank") or 0),
+                                   window=int((m.get("mask") or {}).get("size") or 1 << 30),
                                    rot_dims=int(rot.get("dims", m["rot_dim"])), rot_base=float(rot.get("base", 10000.0)),
                                    scale=float(m["scale"]),
                                    kv_from=(int(m["kv_from"]) if m.get("kv_from") is not None else None))

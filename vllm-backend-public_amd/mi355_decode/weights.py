@@ -445,6 +445,8 @@ def _sandwich_from_getter(cfg: ModelConfig, get, dtype, device) -> ModelWeights:
                       head_norm=f32(expect(m + "norm", (C,))))
         else:
             A = L.lattn
+            if A.q_rank <= 0:                             # not named by the configuration: the tensor's shape gives it
+                A.q_rank = int(get(m + "dq").shape[0])
             parts = [("dq", expect(m + "dq", (A.q_rank, W)))]
             if A.kv_from is None:
                 parts.append(("dkv", expect(m + "dkv", (A.kv_rank + A.rot_dim, W))))
