@@ -391,6 +391,10 @@ def test_routing_groups_corrections_and_negative_choice_scores():
             got = torch.zeros(300, E).scatter_(1, ids.cpu().long(), wts.cpu())
             want = torch.zeros(300, E).scatter_(1, rid, rw)
             assert (got - want).abs().max() < 1e-6
+        z[::7, 1] = float("nan")                              # a NaN logit must not turn into an index outside the experts
+        ids, _ = ops.moe_route(z.cuda(), torch.zeros(E).cuda(), top, count, keep)
+        ids = ids.cpu()
+        assert int(ids.min()) >= 0 and int(ids.max()) < E and all(len(set(r.tolist())) == top for r in ids)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -417,10 +421,10 @@ def test_expert_products_by_rows_and_by_expert_matrices(dtype, T, W, F):
                          down_w=torch.stack([wt[f"e{e}.down"] for e in range(E)]).to(dtype).cuda())
     ff = MoEFeedForward(MoESpec(E, top, 3, 2, F), lw, None)
     tol = 2e-5 if dtype == torch.float32 else 3e-2
-    for min_rows in (1, 1 << 30):                             # one product per expert; the per-row kernels
-        ff.GROUPED_MIN_ROWS = min_rows
+    for min_rows, max_tokens in ((1, 2048), (1 << 30, 2048), (1, 64)):   # products per expert; the per-row kernels; in slices
+        ff.GROUPED_MIN_ROWS, ff.GROUPED_MAX_TOKENS = min_rows, max_tokens
         got = ff(h.cuda()).float().cpu()
-        assert (got - ref).abs().max() <= tol * ref.abs().max(), min_rows
+        assert (got - ref).abs().max() <= tol * ref.abs().max(), (min_rows, max_tokens)
 
 
 # ------------------------------------------------------------------------------------------ #

@@ -100,6 +100,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(int32_t* __restrict
   for (int i = 0; i < EPL; ++i) {
     const int e = lane + 64 * i;
     c[i] = e < E ? 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + e))) + MI355_LD(float, corr, corr + e) : ninf;
+    if (c[i] != c[i]) c[i] = -3.0e38f;                  // a NaN logit ranks last but stays a valid pick: ids are indices downstream
     ch[wave][e] = c[i];
   }
   __syncthreads();

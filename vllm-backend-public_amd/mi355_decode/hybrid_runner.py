@@ -167,7 +167,21 @@ class MoEFeedForward:
     def __init__(self, spec, lw, runner):
         self.s, self.lw, self.r = spec, lw, runner
 
+    GROUPED_MAX_TOKENS = 2048       # longer steps go through the experts in slices of this many tokens
+
     def __call__(self, h: torch.Tensor) -> torch.Tensor:
+        """h [tokens, width] -> the mixture's output, the same shape.  Tokens are independent of each other
+        here, so a long step is served in slices: the padded batched products then stay at sizes where
+        an uneven slice costs little padding, and their temporaries at a few hundred megabytes."""
+        T = h.shape[0]
+        if T <= self.GROUPED_MAX_TOKENS:
+            return self._tokens(h)
+        out = torch.empty_like(h)
+        for a in range(0, T, self.GROUPED_MAX_TOKENS):
+            out[a: a + self.GROUPED_MAX_TOKENS] = self._tokens(h[a: a + self.GROUPED_MAX_TOKENS])
+        return out
+
+    def _tokens(self, h: torch.Tensor) -> torch.Tensor:
         s, lw = self.s, self.lw
         T = h.shape[0]
         ids, wts = ops.moe_route(torch.mm(h.float(), lw.router_w.t()), lw.correction, s.top, s.groups, s.keep)
