@@ -350,11 +350,12 @@ def test_latent_attention_on_the_matrix_cores(H, R_, rot, dims, window):
         assert (got - ref).abs().max() <= 3e-2 * ref.abs().max(), cuts
 
 
-@pytest.mark.parametrize("window", [16, 17, 31, 48, 64, 65])
+@pytest.mark.parametrize("window", [16, 17, 31, 48, 64, 65, 200])
 def test_latent_window_edge_and_sink_show_with_one_loud_key(window):
     """Token 9 holds a latent that every query scores far above all others: a query sees it exactly
-    while 0 <= i - 9 < window; once it is gone the sink, set high, takes most of the weight."""
-    H, R_, rot, T = 2, 32, 8, 9 + 70
+    while 0 <= i - 9 < window (for the widest window: one key among two hundred, a dozen pages back);
+    once it is gone the sink, set high, takes most of the weight."""
+    H, R_, rot, T = 2, 32, 8, 9 + max(70, window + 5)
     g = torch.Generator().manual_seed(window)
     x = torch.randn(T, R_ + rot, generator=g) * 0.1
     x[9, :R_] = 0.0
@@ -370,10 +371,10 @@ def test_latent_window_edge_and_sink_show_with_one_loud_key(window):
     assert float(ref[inside, 0, 3]) > 5.0 and abs(float(ref[outside, 0, 3])) < 2.5     # the edge, in the restatement
     assert float(ref[outside, 0].abs().max()) < 0.3 * float(ref[outside, 1].abs().max())   # the sink takes head 0's weight
     for cuts in ([T], [9 + window - 1, 1, 1] + [1] * 5, [5, 2] + [1] * (T - 7)):
-        got = _latent_in_cuts(x, nw, ql, q, rot, 0, sink, None, cuts, *args)
+        got = _latent_in_cuts(x, nw, ql, q, rot, 0, sink, None, cuts, *args, pages=16)
         assert (got - ref).abs().max() <= 1e-4 * ref.abs().max(), cuts
         b16 = lambda t: t.to(torch.bfloat16)                  # noqa: E731
-        got = _latent_in_cuts(b16(x), nw, b16(ql), b16(q), rot, 0, sink, None, cuts, *args, tiled=True)
+        got = _latent_in_cuts(b16(x), nw, b16(ql), b16(q), rot, 0, sink, None, cuts, *args, pages=16, tiled=True)
         r16 = _latent_ref(b16(x), nw, b16(ql), b16(q), rot, 0, sink, None, *args)
         assert (got - r16).abs().max() <= 3e-2 * r16.abs().max(), cuts
 
@@ -381,7 +382,7 @@ def test_latent_window_edge_and_sink_show_with_one_loud_key(window):
 def test_routing_groups_corrections_and_negative_choice_scores():
     from mi355_decode import ops
     g = torch.Generator().manual_seed(2)
-    for E, top, count, keep in ((8, 2, 2, 1), (12, 3, 4, 2), (6, 1, 6, 2), (16, 4, 1, 1), (9, 9, 3, 3), (64, 8, 8, 4)):
+    for E, top, count, keep in ((8, 2, 2, 1), (12, 3, 4, 2), (6, 1, 6, 2), (16, 4, 1, 1), (9, 9, 3, 3), (64, 8, 8, 4), (160, 20, 5, 3)):
         z = torch.randn(300, E, generator=g) * 2
         # corrections that push every choice score below zero: a barred expert must not beat them as a "0"
         for corr in (torch.randn(E, generator=g) * 0.3, torch.randn(E, generator=g) * 0.3 - 3.0):

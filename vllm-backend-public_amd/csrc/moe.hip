@@ -413,9 +413,10 @@ extern "C" int32_t mi355_moe_route(int32_t* ids, float* weights, const float* lo
   MI355_REQUIRE(num_tokens >= 0 && experts > 0 && top > 0 && groups > 0 && keep > 0 && keep <= groups &&
                     experts % groups == 0,
                 MI355_ERR_INVALID, "moe_route: %d experts in %d groups, %d kept, %d chosen", experts, groups, keep, top);
-  MI355_REQUIRE(top <= kMaxTop && groups <= kMaxGroups && top <= keep * (experts / groups), MI355_ERR_UNSUPPORTED,
-                "moe_route: at most %d chosen experts and %d groups; the kept groups must hold the %d chosen", kMaxTop,
-                kMaxGroups, top);
+  MI355_REQUIRE((top <= kMaxTop || experts <= 512) && groups <= kMaxGroups && top <= keep * (experts / groups),
+                MI355_ERR_UNSUPPORTED,
+                "moe_route: at most %d groups, %d chosen experts of more than 512; the kept groups must hold the %d chosen",
+                kMaxGroups, kMaxTop, top);
   if (num_tokens == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 wgrid(static_cast<unsigned>((num_tokens + 3) / 4));
